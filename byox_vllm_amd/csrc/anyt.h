@@ -22,6 +22,16 @@ __device__ __forceinline__ float silu_f32(float z) { return z / (1.0f + expf(-z)
 __device__ __forceinline__ float gelu_tanh_f32(float z) {
   return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
+// Gated unit act(gate) * up.  act 0: SiLU, 1: tanh-form GELU, 2: the clamped form with limit c,
+// g = min(gate, c), u = clamp(up, -c, c), g * sigmoid(1.702 g) * (u + 1).
+__device__ __forceinline__ float glu_act(float g, float u, int act, float c) {
+  if (act == 2) {
+    g = fminf(g, c);
+    u = fminf(fmaxf(u, -c), c);
+    return g * sigmoid_f32(1.702f * g) * (u + 1.0f);
+  }
+  return (act == 1 ? gelu_tanh_f32(g) : silu_f32(g)) * u;
+}
 // log(sigmoid(z)) without cancellation: -softplus(-z)
 __device__ __forceinline__ float log_sigmoid_f32(float z) {
   return z >= 0.0f ? -log1pf(expf(-z)) : z - log1pf(expf(z));

@@ -166,7 +166,7 @@ __global__ __launch_bounds__(256) void linear_kernel(LinArgs p) {
       if (bias) v += ld_f32<T>(bias + n);
       if constexpr (EPI == EPI_GLU) {
         const float u = accu[i][r];
-        v = (p.act == 1 ? gelu_tanh_f32(v) : silu_f32(v)) * u;
+        v = glu_act(v, u, p.act, p.epi_c);
       } else if constexpr (EPI == EPI_SOFTCAP) {
         v = p.epi_c * tanhf(v / p.epi_c);
       } else if constexpr (EPI == EPI_ROW_GATE) {
@@ -301,7 +301,7 @@ __global__ __launch_bounds__(256) void linear_tile_kernel(LinArgs p) {
         float v = acc[i][j][r];
         if (bias) v += ld_f32<bf16_t>(bias + n);
         if constexpr (GLU) {
-          v = (p.act == 1 ? gelu_tanh_f32(v) : silu_f32(v)) * accu[i][j][r];
+          v = glu_act(v, accu[i][j][r], p.act, p.epi_c);
         } else if constexpr (EPI == EPI_SOFTCAP) {
           v = p.epi_c * tanhf(v / p.epi_c);
         } else if constexpr (EPI == EPI_ROW_GATE) {
@@ -413,7 +413,7 @@ __global__ __launch_bounds__(256) void linear_fewrow_kernel(LinArgs p) {
       if (bias) v += ld_f32<T>(bias + n);
       if constexpr (GLU) {
         const float u = part[1][0][i][e] + part[1][1][i][e] + part[1][2][i][e] + part[1][3][i][e];
-        v = (p.act == 1 ? gelu_tanh_f32(v) : silu_f32(v)) * u;
+        v = glu_act(v, u, p.act, p.epi_c);
       } else if constexpr (EPI == EPI_SOFTCAP) {
         v = p.epi_c * tanhf(v / p.epi_c);
       } else if constexpr (EPI == EPI_ROW_GATE) {

@@ -1,5 +1,6 @@
 // Mixture-of-experts bookkeeping around the grouped products of nv_linear:
-//   nv_moe_route   : per token the `top` largest router logits (fp32) and the softmax over just those
+//   nv_moe_route   : per token the `top` largest router logits (fp32) and the softmax over just those (mode 0), or
+//                    the softmax over all experts, the chosen scores divided by (their sum + 1e-20) (mode 1)
 //   nv_moe_sort    : (token, choice) pairs ordered by expert -> group offsets, the token behind every sorted row and
 //                    the sorted row of every pair
 //   nv_moe_combine : weighted sum of a token's expert rows (+ a sigmoid-gated shared expert)
@@ -9,7 +10,8 @@
 namespace {
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int64_t rs, int E, int top,
-                                                        int32_t* __restrict__ idx, float* __restrict__ wt, int64_t T_) {
+                                                        int32_t* __restrict__ idx, float* __restrict__ wt, int64_t T_,
+                                                        int mode) {
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T_) return;
   const float* row = logits + t * rs;
@@ -31,6 +33,17 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     tw[j] = best;
   }
   const float m = tw[0];   // choices come out in descending order
+  if (mode == 1) {         // scores of the softmax over every expert, renormalised over the chosen ones
+    float all = 0.0f;
+    for (int e = 0; e < E; ++e) all += expf(row[e] - m);
+    float sum = 0.0f;
+    for (int j = 0; j < top; ++j) {
+      tw[j] = expf(tw[j] - m) / all;
+      sum += tw[j];
+    }
+    for (int j = 0; j < top; ++j) tw[j] /= sum + 1e-20f;
+    return;
+  }
   float sum = 0.0f;
   for (int j = 0; j < top; ++j) {
     tw[j] = expf(tw[j] - m);
@@ -70,7 +83,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
                                                           const float* __restrict__ shared, const float* __restrict__ sg,
                                                           int64_t sg_rs, float* __restrict__ out, int width) {
   const int64_t t = blockIdx.x;
-  const float gate = shared ? sigmoid_f32(sg[t * sg_rs]) : 0.0f;
+  const float gate = !shared ? 0.0f : sg ? sigmoid_f32(sg[t * sg_rs]) : 1.0f;   // no gate logits: a plain addend
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     float a = 0.0f;
     for (int j = 0; j < top; ++j) a += wt[t * top + j] * y[(int64_t)slot_of[t * top + j] * width + c];
@@ -82,13 +95,14 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 }  // namespace
 
 extern "C" int nv_moe_route(const float* logits, int64_t row_stride, int32_t* idx, float* weights, int64_t tokens,
-                            int experts, int top, nv_stream_t stream) {
+                            int experts, int top, int mode, nv_stream_t stream) {
   NV_CHECK_ARG(logits && idx && weights, "nv_moe_route: null pointer");
+  NV_CHECK_ARG(mode == 0 || mode == 1, "nv_moe_route: bad mode %d", mode);
   NV_CHECK_ARG(tokens >= 0 && experts > 0 && top > 0 && top <= experts, "nv_moe_route: bad shape experts=%d top=%d",
                experts, top);
   if (tokens == 0) return NV_OK;
   moe_route_kernel<<<dim3((unsigned)((tokens + 255) / 256)), dim3(256), 0, (hipStream_t)stream>>>(
-      logits, row_stride, experts, top, idx, weights, tokens);
+      logits, row_stride, experts, top, idx, weights, tokens, mode);
   NV_CHECK_LAUNCH();
   return NV_OK;
 }
@@ -107,7 +121,6 @@ extern "C" int nv_moe_combine(const float* y, const int32_t* slot_of, const floa
                               const float* shared_gate, int64_t shared_gate_stride, float* out, int64_t tokens,
                               int width, nv_stream_t stream) {
   NV_CHECK_ARG(y && slot_of && weights && out, "nv_moe_combine: null pointer");
-  NV_CHECK_ARG(!shared || shared_gate, "nv_moe_combine: a shared expert needs its gate logits");
   NV_CHECK_ARG(tokens >= 0 && top > 0 && width > 0, "nv_moe_combine: bad shape");
   if (tokens == 0) return NV_OK;
   moe_combine_kernel<<<dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream>>>(y, slot_of, weights, top, shared,

@@ -51,15 +51,32 @@ __global__ __launch_bounds__(256) void rmsnorm_f32_kernel(const float* __restric
   for (int j = threadIdx.x; j < n; j += blockDim.x) st_f32<T>(out + r * out_rs + j, xr[j] * inv * ld_f32<T>(w + j));
 }
 
+// out[t] = [x[t] | x0[t]] in the storage type; x takes delta first
+template <typename T>
+__global__ __launch_bounds__(256) void residual_pair_kernel(float* __restrict__ x, const float* __restrict__ delta,
+                                                            int64_t delta_rs, const float* __restrict__ x0,
+                                                            T* __restrict__ out, int n) {
+  const int64_t t = blockIdx.x;
+  for (int j = threadIdx.x; j < n; j += blockDim.x) {
+    float v = x[t * n + j];
+    if (delta) {
+      v += delta[t * delta_rs + j];
+      x[t * n + j] = v;
+    }
+    st_f32<T>(out + t * 2 * n + j, v);
+    st_f32<T>(out + t * 2 * n + n + j, x0[t * n + j]);
+  }
+}
+
 // out[m][j] = act(y[m][j]) * y[m][n + j]: the gated unit's activation over a plain product's [gate | up] rows
 template <typename T>
 __global__ __launch_bounds__(256) void act_mul_f32_kernel(const float* __restrict__ y, T* __restrict__ out, int64_t total,
-                                                          int n, int act) {
+                                                          int n, int act, float c) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t m = i / n;
     const int j = (int)(i - m * n);
     const float g = y[m * 2 * n + j], u = y[m * 2 * n + n + j];
-    st_f32<T>(out + i, (act == 1 ? gelu_tanh_f32(g) : silu_f32(g)) * u);
+    st_f32<T>(out + i, glu_act(g, u, act, c));
   }
 }
 
@@ -144,16 +161,29 @@ extern "C" int nv_sample_f32(const float* logits, int64_t row_stride, const floa
   return NV_OK;
 }
 
-extern "C" int nv_act_mul_f32(const float* y, void* out, int64_t rows, int n, int act, int dtype, nv_stream_t stream) {
+extern "C" int nv_residual_pair(float* x, const float* delta, int64_t delta_row_stride, const float* x0, void* out,
+                                int64_t rows, int n, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(x && x0 && out, "nv_residual_pair: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_residual_pair: bad dtype %d", dtype);
+  NV_CHECK_ARG(rows >= 0 && rows < (1ll << 31) && n > 0, "nv_residual_pair: bad shape");
+  if (rows == 0) return NV_OK;
+  NV_DISPATCH_T(dtype, residual_pair_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
+                           x, delta, delta_row_stride, x0, (T*)out, n));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_act_mul_f32(const float* y, void* out, int64_t rows, int n, int act, float c, int dtype,
+                              nv_stream_t stream) {
   NV_CHECK_ARG(y && out, "nv_act_mul_f32: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_act_mul_f32: bad dtype %d", dtype);
-  NV_CHECK_ARG(rows >= 0 && n > 0 && (act == 0 || act == 1), "nv_act_mul_f32: bad shape or activation");
+  NV_CHECK_ARG(rows >= 0 && n > 0 && act >= 0 && act <= 2 && (act != 2 || c > 0.0f), "nv_act_mul_f32: bad shape or activation");
   if (rows == 0) return NV_OK;
   const int64_t total = rows * n;
   int64_t blocks = (total + 255) / 256;
   if (blocks > 8192) blocks = 8192;
   NV_DISPATCH_T(dtype, act_mul_f32_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
-                           y, (T*)out, total, n, act));
+                           y, (T*)out, total, n, act, c));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

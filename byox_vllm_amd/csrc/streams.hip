@@ -138,11 +138,13 @@ __global__ __launch_bounds__(256) void token_shift_kernel(const float* __restric
   }
 }
 
-// rows of `groups` equal parts, each divided by its own root mean square and multiplied by its slice of w
+// rows of `groups` equal parts, each divided by its own root mean square and multiplied by its slice of w (and, with
+// gate logits of the same layout, by their sigmoid)
 template <typename T>
 __global__ __launch_bounds__(256) void group_rmsnorm_f32_kernel(const float* __restrict__ x, int64_t x_rs,
                                                                 const T* __restrict__ w, T* __restrict__ out,
-                                                                int64_t out_rs, int groups, int n, float eps) {
+                                                                int64_t out_rs, int groups, int n, float eps,
+                                                                const float* __restrict__ gate, int64_t gate_rs) {
   __shared__ float red[32];
   const int64_t t = blockIdx.x / groups;
   const int g = blockIdx.x % groups;
@@ -151,8 +153,11 @@ __global__ __launch_bounds__(256) void group_rmsnorm_f32_kernel(const float* __r
   for (int j = threadIdx.x; j < n; j += blockDim.x) ss += xr[j] * xr[j];
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)n + eps);
-  for (int j = threadIdx.x; j < n; j += blockDim.x)
-    st_f32<T>(out + t * out_rs + (int64_t)g * n + j, xr[j] * inv * ld_f32<T>(w + (int64_t)g * n + j));
+  for (int j = threadIdx.x; j < n; j += blockDim.x) {
+    float v = xr[j] * inv * ld_f32<T>(w + (int64_t)g * n + j);
+    if (gate) v *= sigmoid_f32(gate[t * gate_rs + (int64_t)g * n + j]);
+    st_f32<T>(out + t * out_rs + (int64_t)g * n + j, v);
+  }
 }
 
 }  // namespace
@@ -213,13 +218,14 @@ extern "C" int nv_token_shift(const float* h, const void* mu, float* state, cons
 }
 
 extern "C" int nv_group_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* out, int64_t out_row_stride,
-                                    int64_t rows, int groups, int n, float eps, int dtype, nv_stream_t stream) {
+                                    int64_t rows, int groups, int n, float eps, const float* gate,
+                                    int64_t gate_row_stride, int dtype, nv_stream_t stream) {
   NV_CHECK_ARG(x && w && out, "nv_group_rmsnorm_f32: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_group_rmsnorm_f32: bad dtype %d", dtype);
   NV_CHECK_ARG(rows >= 0 && n > 0 && groups > 0 && rows * groups < (1ll << 31), "nv_group_rmsnorm_f32: bad shape");
   if (rows == 0) return NV_OK;
   NV_DISPATCH_T(dtype, group_rmsnorm_f32_kernel<T><<<dim3((unsigned)(rows * groups)), dim3(256), 0, (hipStream_t)stream>>>(
-                           x, x_row_stride, (const T*)w, (T*)out, out_row_stride, groups, n, eps));
+                           x, x_row_stride, (const T*)w, (T*)out, out_row_stride, groups, n, eps, gate, gate_row_stride));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

@@ -3,11 +3,14 @@
 //     s_ij = cap(q_i . k_j) - slope_h (i - j),   cap(z) = c tanh(z / c) (or z without a cap),
 // over the keys 0 <= i - j < window (window 0: every earlier key).  q arrives already normalised and multiplied by its
 // scale and per-head temperature (qk_norm_store below), so the kernel's own arithmetic is the dot product, the cap,
-// the distance term and the softmax, all in fp32.
+// the distance term and the softmax, all in fp32.  Options of a design: no distance term; a sink, one learned logit per
+// query head that joins the softmax's denominator without a key or a value; values that ARE the keys (rows [k: G * d]
+// only, read twice); a sigmoid output gate from fp32 logits laid out like the output.
 //
 // qk_norm_store: per token, RMS norm over each query and key head (one weight vector shared by the heads), the query
 // scaled by scale * temp[h] and left in fp32, the normalised key and the value written to the token's cache row
-// [k: G * d | v: G * dv] in the storage type.
+// [k: G * d | v: G * dv] in the storage type.  The norms may be absent (null weights: the projection as it is), and
+// the query may carry a temperature that grows with the position p: 1 + coef * ln(floor((p + 1) / every) + 1).
 //
 // window_attn_kernel: a workgroup owns TQ consecutive tokens of the packed batch and one key/value head, i.e. up to
 // TQ * (H / G) query rows that read the same keys; tokens of different requests inside the tile are served one request
@@ -24,6 +27,9 @@ struct QkArgs {
   const void* qn;         // [d] query norm weight
   const void* kn;         // [d]
   const void* temp;       // [H] or null
+  const int64_t* positions;   // [tokens], read when temp_every > 0
+  float temp_coef;
+  int temp_every;         // 0: no position temperature
   const int32_t* slot_mapping;   // [tokens] cache row of each token, -1: none
   void* cache;            // [rows, G * (d + dv)]
   float* q_out;           // [tokens, H * d]
@@ -37,8 +43,10 @@ __global__ __launch_bounds__(256) void qk_norm_store_kernel(QkArgs p) {
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const float* row = p.proj + t * p.proj_rs;
   const int64_t slot = p.slot_mapping[t];
-  const int cw = p.G * (p.d + p.dv);
+  const int cw = p.G * (p.d + p.dv);       // dv 0: the values are the keys, rows hold keys only
   T* crow = slot >= 0 ? reinterpret_cast<T*>(p.cache) + slot * cw : nullptr;
+  float pos_temp = 1.0f;
+  if (p.temp_every > 0) pos_temp = 1.0f + p.temp_coef * logf((float)((p.positions[t] + 1) / p.temp_every) + 1.0f);
   const T* qn = reinterpret_cast<const T*>(p.qn);
   const T* kn = reinterpret_cast<const T*>(p.kn);
   const T* temp = reinterpret_cast<const T*>(p.temp);
@@ -47,27 +55,30 @@ __global__ __launch_bounds__(256) void qk_norm_store_kernel(QkArgs p) {
     const bool is_q = v < p.H;
     const int col = is_q ? p.q_off + v * p.d : p.k_off + (v - p.H) * p.d;
     const float* src = row + col;
-    float ss = 0.0f;
-    for (int e = lane; e < p.d; e += 64) {
-      const float x = src[e] + (bias ? ld_f32<T>(bias + col + e) : 0.0f);
-      ss += x * x;
-    }
-    ss = wave_sum(ss);
-    const float inv = 1.0f / sqrtf(ss / (float)p.d + p.eps);
-    if (is_q) {
-      const float f = p.scale * (temp ? ld_f32<T>(temp + v) : 1.0f);
+    float inv = 1.0f;
+    if (qn) {
+      float ss = 0.0f;
       for (int e = lane; e < p.d; e += 64) {
         const float x = src[e] + (bias ? ld_f32<T>(bias + col + e) : 0.0f);
-        p.q_out[t * p.H * p.d + v * p.d + e] = x * inv * ld_f32<T>(qn + e) * f;
+        ss += x * x;
+      }
+      ss = wave_sum(ss);
+      inv = 1.0f / sqrtf(ss / (float)p.d + p.eps);
+    }
+    if (is_q) {
+      const float f = p.scale * (temp ? ld_f32<T>(temp + v) : 1.0f) * pos_temp;
+      for (int e = lane; e < p.d; e += 64) {
+        const float x = src[e] + (bias ? ld_f32<T>(bias + col + e) : 0.0f);
+        p.q_out[t * p.H * p.d + v * p.d + e] = x * inv * (qn ? ld_f32<T>(qn + e) : 1.0f) * f;
       }
     } else if (crow) {
       for (int e = lane; e < p.d; e += 64) {
         const float x = src[e] + (bias ? ld_f32<T>(bias + col + e) : 0.0f);
-        st_f32<T>(crow + (v - p.H) * p.d + e, x * inv * ld_f32<T>(kn + e));
+        st_f32<T>(crow + (v - p.H) * p.d + e, x * inv * (kn ? ld_f32<T>(kn + e) : 1.0f));
       }
     }
   }
-  if (crow)
+  if (crow && p.dv > 0)
     for (int e = threadIdx.x; e < p.G * p.dv; e += blockDim.x)
       st_f32<T>(crow + p.G * p.d + e, row[p.v_off + e] + (bias ? ld_f32<T>(bias + p.v_off + e) : 0.0f));
 }
@@ -85,7 +96,24 @@ struct WAttnArgs {
   int64_t tokens;
   int H, G, d, dv, block_size, window, TQ, TK;
   float softcap, out_scale;
+  int cw, v_col;           // numbers per cache row; column where the values of key/value head 0 begin (0: the keys)
+  int slope_on;            // the distance term 2^(-8 (h + 1) / H) (i - j)
+  const void* sink;        // [H] logits that join the denominator, or null
+  const float* gate;       // [tokens, gate_rs] logits whose sigmoid multiplies the output (head h at h * dv), or null
+  int64_t gate_rs;
 };
+
+// (factor for the accumulated values, denominator) once the walk over the keys is over: the sink joins the sum
+__device__ __forceinline__ void close_softmax(float m, float l, bool has_sink, float sink, float& f, float& den) {
+  if (!has_sink) {
+    f = 1.0f;
+    den = l;
+    return;
+  }
+  const float top = fmaxf(m, sink);
+  f = m == -INFINITY ? 0.0f : expf(m - top);
+  den = l * f + expf(sink - top);
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void window_attn_kernel(WAttnArgs p) {
@@ -105,8 +133,9 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WAttnArgs p) {
   const int64_t t_begin = (int64_t)blockIdx.x * p.TQ;
   const int64_t t_end = min(p.tokens, t_begin + p.TQ);
   const T* cache = reinterpret_cast<const T*>(p.cache);
-  const int cw = p.G * (d + dv);
+  const int cw = p.cw;
   T* out = reinterpret_cast<T*>(p.out);
+  const T* sink = reinterpret_cast<const T*>(p.sink);
 
   for (int64_t ts = t_begin; ts < t_end;) {
     const int b = p.seq_of[ts];
@@ -132,7 +161,7 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WAttnArgs p) {
         const int kp = j0 + j;
         const int64_t crow = (int64_t)table[kp / p.block_size] * p.block_size + kp % p.block_size;
         if (e < d) sk[j * dp + e] = ld_f32<T>(cache + crow * cw + g * d + e);
-        else sv[j * dv + e - d] = ld_f32<T>(cache + crow * cw + p.G * d + g * dv + e - d);
+        else sv[j * dv + e - d] = ld_f32<T>(cache + crow * cw + p.v_col + g * dv + e - d);
       }
       __syncthreads();
       for (int i = tid; i < rows * TK; i += 256) {
@@ -146,7 +175,7 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WAttnArgs p) {
           for (int e = 0; e < d; ++e) s += qv[e] * kv[e];
           if (p.softcap > 0.0f) s = p.softcap * tanhf(s / p.softcap);
           const int h = g * R + rr % R;
-          s -= exp2f(-8.0f * (float)(h + 1) / (float)p.H) * (float)(pos - kp);
+          if (p.slope_on) s -= exp2f(-8.0f * (float)(h + 1) / (float)p.H) * (float)(pos - kp);
         }
         sc[i] = s;
       }
@@ -183,8 +212,12 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WAttnArgs p) {
       __syncthreads();
     }
     for (int i = tid; i < rows * dv; i += 256) {
-      const int rr = i / dv, e = i % dv;
-      st_f32<T>(out + (ts + rr / R) * p.out_rs + (g * R + rr % R) * dv + e, acc[i] / sl[rr] * p.out_scale);
+      const int rr = i / dv, e = i % dv, h = g * R + rr % R;
+      float f, den;
+      close_softmax(sm[rr], sl[rr], sink != nullptr, sink ? ld_f32<T>(sink + h) : 0.0f, f, den);
+      float v = acc[i] * f / den * p.out_scale;
+      if (p.gate) v *= sigmoid_f32(p.gate[(ts + rr / R) * p.gate_rs + h * dv + e]);
+      st_f32<T>(out + (ts + rr / R) * p.out_rs + h * dv + e, v);
     }
     __syncthreads();
     ts = te;
@@ -242,8 +275,9 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
   const int64_t t_begin = (int64_t)blockIdx.x * p.TQ;
   const int64_t t_end = min(p.tokens, t_begin + p.TQ);
   const bf16_t* cache = reinterpret_cast<const bf16_t*>(p.cache);
-  const int cw = p.G * (d + dv);
+  const int cw = p.cw;
   bf16_t* out = reinterpret_cast<bf16_t*>(p.out);
+  const bf16_t* sink = reinterpret_cast<const bf16_t*>(p.sink);
 
   for (int64_t ts = t_begin; ts < t_end;) {
     const int b = p.seq_of[ts];
@@ -276,7 +310,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
       const int rr = row0 + lg * 4 + r;
       valid[r] = rr < rows;
       pos[r] = p0 + rr / R;
-      slope[r] = exp2f(-8.0f * (float)(g * R + rr % R + 1) / (float)p.H);
+      slope[r] = p.slope_on ? exp2f(-8.0f * (float)(g * R + rr % R + 1) / (float)p.H) : 0.0f;
       m_run[r] = -INFINITY;
       l_run[r] = 0.0f;
     }
@@ -307,7 +341,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
         const int64_t row = sRow[key];
         vreg[i] = u32x4{0u, 0u, 0u, 0u};
         if (row >= 0 && part * 8 < dv)
-          vreg[i] = *reinterpret_cast<const u32x4*>(cache + row * cw + p.G * d + g * dv + part * 8);
+          vreg[i] = *reinterpret_cast<const u32x4*>(cache + row * cw + p.v_col + g * dv + part * 8);
       }
 #pragma unroll
       for (int i = 0; i < NKC; ++i) {
@@ -422,7 +456,12 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
           l += pw[rr * PW + DVP + 1] * f;
           o += pw[rr * PW + e] * f;
         }
-        out[(ts + rr / R) * p.out_rs + (g * R + rr % R) * dv + e] = (bf16_t)(o * p.out_scale / l);
+        const int h = g * R + rr % R;
+        float f, den;
+        close_softmax(m, l, sink != nullptr, sink ? ld_f32<bf16_t>(sink + h) : 0.0f, f, den);
+        float v = o * f * p.out_scale / den;
+        if (p.gate) v *= sigmoid_f32(p.gate[(ts + rr / R) * p.gate_rs + h * dv + e]);
+        out[(ts + rr / R) * p.out_rs + h * dv + e] = (bf16_t)v;
       }
       __syncthreads();
     } else if (wave_on) {
@@ -430,12 +469,16 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
       for (int r = 0; r < 4; ++r) {
         const int rr = row0 + lg * 4 + r;
         if (!valid[r]) continue;
-        const float f = p.out_scale / l_run[r];
-        bf16_t* orow = out + (ts + rr / R) * p.out_rs + (g * R + rr % R) * dv;
+        const int h = g * R + rr % R;
+        float fs, den;
+        close_softmax(m_run[r], l_run[r], sink != nullptr, sink ? ld_f32<bf16_t>(sink + h) : 0.0f, fs, den);
+        const float f = p.out_scale * fs / den;
+        bf16_t* orow = out + (ts + rr / R) * p.out_rs + h * dv;
+        const float* grow = p.gate ? p.gate + (ts + rr / R) * p.gate_rs + h * dv : nullptr;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
           const int e = ct * 16 + lc;
-          if (e < dv) orow[e] = (bf16_t)(acc_o[ct][r] * f);
+          if (e < dv) orow[e] = (bf16_t)(acc_o[ct][r] * f * (grow ? sigmoid_f32(grow[e]) : 1.0f));
         }
       }
     }
@@ -477,27 +520,52 @@ hipError_t launch_window_mfma(const WAttnArgs& p, int ct, bool split, dim3 grid,
 
 }  // namespace
 
+extern "C" int nv_qk_store(const float* proj, const void* bias, int64_t proj_row_stride, int q_off, int k_off, int v_off,
+                           const void* q_norm, const void* k_norm, const void* temp, const int64_t* positions,
+                           float temp_coef, int temp_every, float scale, float eps, const int32_t* slot_mapping,
+                           void* cache, float* q_out, int64_t tokens, int heads, int kv_heads, int dim, int vdim, int dtype,
+                           nv_stream_t stream) {
+  NV_CHECK_ARG(proj && slot_mapping && cache && q_out, "nv_qk_store: null pointer");
+  NV_CHECK_ARG((q_norm == nullptr) == (k_norm == nullptr), "nv_qk_store: both norm weights or none");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_qk_store: bad dtype %d", dtype);
+  NV_CHECK_ARG(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim >= 0,
+               "nv_qk_store: bad shape");
+  NV_CHECK_ARG(temp_every >= 0 && (temp_every == 0 || positions), "nv_qk_store: the position temperature needs positions");
+  if (tokens == 0) return NV_OK;
+  QkArgs p{proj, bias, proj_row_stride, q_off, k_off, v_off, q_norm, k_norm, temp, positions, temp_coef, temp_every,
+           slot_mapping, cache, q_out, heads, kv_heads, dim, vdim, scale, eps};
+  NV_DISPATCH_T(dtype, qk_norm_store_kernel<T><<<dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream>>>(p));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
 extern "C" int nv_qk_norm_store(const float* proj, const void* bias, int64_t proj_row_stride, int q_off, int k_off,
                                 int v_off, const void* q_norm, const void* k_norm, const void* temp, float scale, float eps,
                                 const int32_t* slot_mapping, void* cache, float* q_out, int64_t tokens, int heads,
                                 int kv_heads, int dim, int vdim, int dtype, nv_stream_t stream) {
-  NV_CHECK_ARG(proj && q_norm && k_norm && slot_mapping && cache && q_out, "nv_qk_norm_store: null pointer");
-  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_qk_norm_store: bad dtype %d", dtype);
-  NV_CHECK_ARG(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0,
-               "nv_qk_norm_store: bad shape");
-  if (tokens == 0) return NV_OK;
-  QkArgs p{proj, bias, proj_row_stride, q_off, k_off, v_off, q_norm, k_norm, temp, slot_mapping, cache, q_out, heads, kv_heads,
-           dim, vdim, scale, eps};
-  NV_DISPATCH_T(dtype, qk_norm_store_kernel<T><<<dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream>>>(p));
-  NV_CHECK_LAUNCH();
-  return NV_OK;
+  NV_CHECK_ARG(q_norm && k_norm && vdim > 0, "nv_qk_norm_store: null pointer");
+  return nv_qk_store(proj, bias, proj_row_stride, q_off, k_off, v_off, q_norm, k_norm, temp, nullptr, 0.0f, 0, scale, eps,
+                     slot_mapping, cache, q_out, tokens, heads, kv_heads, dim, vdim, dtype, stream);
 }
 
 extern "C" int nv_window_attn(const float* q, const void* cache, const int32_t* block_tables, int table_cols,
                               const int32_t* cu_q, const int32_t* past_lens, const int32_t* seq_of_token, void* out,
                               int64_t out_row_stride, int64_t tokens, int max_q, int heads, int kv_heads, int dim, int vdim,
                               int block_size, int window, float softcap, float out_scale, int dtype, nv_stream_t stream) {
+  return nv_paged_softmax_attn(q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride,
+                               tokens, max_q, heads, kv_heads, dim, vdim, block_size, window, softcap, out_scale, 1, 0,
+                               nullptr, nullptr, 0, dtype, stream);
+}
+
+extern "C" int nv_paged_softmax_attn(const float* q, const void* cache, const int32_t* block_tables, int table_cols,
+                                     const int32_t* cu_q, const int32_t* past_lens, const int32_t* seq_of_token, void* out,
+                                     int64_t out_row_stride, int64_t tokens, int max_q, int heads, int kv_heads, int dim,
+                                     int vdim, int block_size, int window, float softcap, float out_scale, int distance_term,
+                                     int values_are_keys, const void* sink, const float* gate, int64_t gate_row_stride,
+                                     int dtype, nv_stream_t stream) {
   NV_CHECK_ARG(q && cache && block_tables && cu_q && past_lens && seq_of_token && out, "nv_window_attn: null pointer");
+  NV_CHECK_ARG(!values_are_keys || vdim == dim, "nv_window_attn: values that are the keys have the keys' size");
+  const int cw = values_are_keys ? kv_heads * dim : kv_heads * (dim + vdim), v_col = values_are_keys ? 0 : kv_heads * dim;
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_window_attn: bad dtype %d", dtype);
   NV_CHECK_ARG(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 &&
                    block_size > 0 && window >= 0 && table_cols > 0,
@@ -506,14 +574,15 @@ extern "C" int nv_window_attn(const float* q, const void* cache, const int32_t* 
   const int R = heads / kv_heads;
   // bf16 caches with 16-byte-aligned heads of up to 256 numbers: the matrix-core kernel
   if (dtype == NV_BF16 && dim % 8 == 0 && vdim % 8 == 0 && dim <= 256 && vdim <= 256 && R <= 64 && kv_heads <= 65535 &&
-      (uintptr_t)cache % 16 == 0 && getenv("NV_WINDOW_ATTN_MFMA_OFF") == nullptr) {
+      (uintptr_t)cache % 16 == 0 && cw % 8 == 0 && v_col % 8 == 0 && getenv("NV_WINDOW_ATTN_MFMA_OFF") == nullptr) {
     const int ks = dim <= 64 ? 2 : dim <= 128 ? 4 : 8;
     const int ct = vdim <= 32 ? 2 : vdim <= 64 ? 4 : vdim <= 128 ? 8 : 16;
     if (ma_lds_bytes(ks, ct, false) <= 160 * 1024) {
       const bool split = max_q <= 1 && R <= 16;           // one token per request: the wavefronts split the window
       const int TQm = max_q <= 1 ? 1 : 64 / R;
       WAttnArgs pm{q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride, tokens, heads,
-                   kv_heads, dim, vdim, block_size, window, TQm, MA_KEYS, softcap, out_scale};
+                   kv_heads, dim, vdim, block_size, window, TQm, MA_KEYS, softcap, out_scale, cw, v_col, distance_term, sink,
+                   gate, gate_row_stride};
       dim3 gridm((unsigned)((tokens + TQm - 1) / TQm), (unsigned)kv_heads);
       hipStream_t st = (hipStream_t)stream;
       const hipError_t e = ks == 2 ? launch_window_mfma<2>(pm, ct, split, gridm, st)
@@ -538,7 +607,8 @@ extern "C" int nv_window_attn(const float* q, const void* cache, const int32_t* 
   NV_CHECK_ARG(R <= 256 && kv_heads <= 65535, "nv_window_attn: %d query heads per key head exceed a workgroup", R);
   const int64_t tiles = (tokens + TQ - 1) / TQ;
   WAttnArgs p{q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride, tokens, heads,
-              kv_heads, dim, vdim, block_size, window, TQ, TK, softcap, out_scale};
+              kv_heads, dim, vdim, block_size, window, TQ, TK, softcap, out_scale, cw, v_col, distance_term, sink, gate,
+              gate_row_stride};
   dim3 grid((unsigned)tiles, (unsigned)kv_heads);
   NV_DISPATCH_T(dtype, window_attn_kernel<T><<<grid, dim3(256), need(TQ, TK), (hipStream_t)stream>>>(p));
   NV_CHECK_LAUNCH();

@@ -438,6 +438,8 @@ def stage_decode_packed(packed, bs, bt_cols, g, prev_tokens=None, block_size=0):
 
 EPI_NONE, EPI_GLU, EPI_SOFTCAP, EPI_ROW_GATE, EPI_ACT = 0, 1, 2, 3, 4
 ACT_SILU, ACT_GELU_TANH, ACT_XIELU, ACT_SCALE = 0, 1, 2, 3
+GLU_CLAMPED = 2      # EPI_GLU only: g sigmoid(1.702 g) (u + 1) with g = min(gate, cap), u = clamp(up, -cap, cap)
+ROUTE_CHOSEN, ROUTE_ALL = 0, 1   # softmax over the chosen logits / over every expert, renormalised over the chosen
 
 
 def _code32(dt) -> int:
@@ -466,7 +468,7 @@ def linear(x, w, bias=None, out=None, out_dtype=None, *, rows=None, a_rows=None,
         if epilogue == EPI_GLU:      # [gate | up] rows from the library, activation and product in one pass over them
             y = _linear_many_rows(x, w, M, 2 * n, K, torch.float32)
             out = torch.empty(M, n, dtype=out_dtype or x.dtype, device=x.device)
-            check(lib().nv_act_mul_f32(ptr(y), ptr(out), M, n, act, _code32(out.dtype), stream()), "nv_act_mul_f32")
+            check(lib().nv_act_mul_f32(ptr(y), ptr(out), M, n, act, cap, _code32(out.dtype), stream()), "nv_act_mul_f32")
             return out
         if epilogue == EPI_ACT:      # the element-wise function in one pass over the library's fp32 result
             y = _linear_many_rows(x, w, M, n, K, torch.float32)
@@ -577,6 +579,61 @@ def gla_recurrent(proj, offsets, z, state, cu_q, past_lens, state_slots, norm_w,
     return out
 
 
+MEM_CONST, MEM_EXPGATE = 0, 1
+
+
+def matrix_memory_state_size(mode, dim, vdim) -> int:
+    """fp32 numbers one head keeps between steps: the matrix, and in the gated form the normaliser and the maximum."""
+    return dim * vdim + (dim + 1 if mode == MEM_EXPGATE else 0)
+
+
+def matrix_memory(proj, offsets, state, cu_q, past_lens, state_slots, heads, dim, vdim, mode, *, decay=None, bias=None,
+                  gate_offsets=(0, 0), cap=0.0, silu=False, q_scale=1.0, out=None):
+    """Matrix memory with one decay per head and token over the step's tokens; ``proj`` fp32 [T, *] holds q | k | v at
+    ``offsets`` (and, MEM_EXPGATE, one input-gate and one forget-gate logit per head at ``gate_offsets``, to which
+    ``bias`` over proj's columns is added); ``state`` fp32 [slots, heads, state size] is read (unless the request
+    starts) and written back.  -> fp32 [T, heads * vdim]."""
+    require_gpu(proj, "matrix_memory")
+    T = proj.size(0)
+    assert proj.dtype == state.dtype == torch.float32 and proj.stride(1) == 1 and state.is_contiguous()
+    assert state.shape[1:] == (heads, matrix_memory_state_size(mode, dim, vdim))
+    assert cu_q.dtype == past_lens.dtype == state_slots.dtype == torch.int32
+    B = past_lens.numel()
+    assert cu_q.numel() == B + 1 and state_slots.numel() == B
+    q_off, k_off, v_off = offsets
+    i_off, f_off = gate_offsets
+    cols = proj.size(1)
+    assert max(q_off + heads * dim, k_off + heads * dim, v_off + heads * vdim) <= cols
+    dt = torch.float32
+    if mode == MEM_CONST:
+        assert decay is not None and decay.dtype == torch.float32 and decay.numel() == heads and decay.is_cuda
+    else:
+        assert max(i_off, f_off) + heads <= cols and cap > 0
+        if bias is not None:
+            assert bias.is_contiguous() and bias.numel() >= max(i_off, f_off) + heads and bias.is_cuda
+            dt = bias.dtype
+    out = torch.empty(T, heads * vdim, dtype=torch.float32, device=proj.device) if out is None else out
+    assert out.dtype == torch.float32 and out.stride(1) == 1 and out.size(0) == T and out.size(1) >= heads * vdim
+    check(lib().nv_matrix_memory(ptr(proj), proj.stride(0), q_off, k_off, v_off, i_off, f_off, ptr(bias), ptr(decay),
+                                 ptr(state), ptr(cu_q), ptr(past_lens), ptr(state_slots), ptr(out), out.stride(0), B, heads,
+                                 dim, vdim, mode, int(silu), q_scale, cap, _code32(dt), stream()), "nv_matrix_memory")
+    return out
+
+
+def residual_pair(x, x0, dtype, delta=None):
+    """[x | x0] rows in ``dtype`` for the projection that re-enters a block of layers; the fp32 rows ``x`` take ``delta``
+    in place first."""
+    require_gpu(x, "residual_pair")
+    assert x.dtype == x0.dtype == torch.float32 and x.is_contiguous() and x0.is_contiguous() and x.shape == x0.shape
+    assert x.dim() == 2
+    if delta is not None:
+        assert delta.dtype == torch.float32 and delta.stride(1) == 1 and delta.shape == x.shape
+    out = torch.empty(x.size(0), 2 * x.size(1), dtype=dtype, device=x.device)
+    check(lib().nv_residual_pair(ptr(x), ptr(delta), delta.stride(0) if delta is not None else 0, ptr(x0), ptr(out),
+                                 x.size(0), x.size(1), _code32(dtype), stream()), "nv_residual_pair")
+    return out
+
+
 def latent_kv_store(kv, norm_w, positions, inv_freq, mscale, slot_mapping, cache, rank, rot_dim, rot_dims, eps):
     require_gpu(kv, "latent_kv_store")
     assert kv.dtype == torch.float32 and kv.stride(1) == 1 and kv.size(1) == rank + rot_dim
@@ -613,14 +670,16 @@ def latent_attn(qa, cache, block_tables, cu_q, past_lens, seq_of_token, heads, r
     return out
 
 
-def moe_route(logits, experts, top):
-    """fp32 router logits [T, >=experts] -> (chosen experts int32 [T, top], softmax over the chosen logits fp32 [T, top])."""
+def moe_route(logits, experts, top, mode=ROUTE_CHOSEN):
+    """fp32 router logits [T, >=experts] -> (chosen experts int32 [T, top], their weights fp32 [T, top]): the softmax
+    over the chosen logits, or (ROUTE_ALL) scores of the softmax over all experts divided by the chosen ones' sum."""
     require_gpu(logits, "moe_route")
     assert logits.dtype == torch.float32 and logits.stride(1) == 1
     T = logits.size(0)
     idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
     wt = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-    check(lib().nv_moe_route(ptr(logits), logits.stride(0), ptr(idx), ptr(wt), T, experts, top, stream()), "nv_moe_route")
+    check(lib().nv_moe_route(ptr(logits), logits.stride(0), ptr(idx), ptr(wt), T, experts, top, mode, stream()),
+          "nv_moe_route")
     return idx, wt
 
 
@@ -641,7 +700,8 @@ def moe_combine(y, slot_of, weights, shared=None, shared_gate=None, out=None):
     width = y.size(1)
     assert y.dtype == weights.dtype == torch.float32 and y.is_contiguous() and weights.is_contiguous()
     if shared is not None:
-        assert shared.dtype == torch.float32 and shared.is_contiguous() and shared_gate.dtype == torch.float32
+        assert shared.dtype == torch.float32 and shared.is_contiguous() and shared.shape == (T, width)
+        assert shared_gate is None or shared_gate.dtype == torch.float32
     out = torch.empty(T, width, dtype=torch.float32, device=y.device) if out is None else out
     check(lib().nv_moe_combine(ptr(y), ptr(slot_of), ptr(weights), top, ptr(shared), ptr(shared_gate),
                                shared_gate.stride(0) if shared_gate is not None else 0, ptr(out), T, width, stream()),
@@ -701,14 +761,17 @@ def token_shift(h, mu, state, cu_q, past_lens, state_slots, seq_of_token, out=No
     return out
 
 
-def group_rms_norm_f32(x, w, groups, eps, out=None):
-    """fp32 rows [T, groups * n]: every part of n numbers by its own root mean square, times w -> rows in w's dtype."""
+def group_rms_norm_f32(x, w, groups, eps, out=None, gate=None):
+    """fp32 rows [T, groups * n]: every part of n numbers by its own root mean square, times w (times sigmoid of the
+    fp32 ``gate`` logits of the same layout, if given) -> rows in w's dtype."""
     require_gpu(x, "group_rms_norm_f32")
     assert x.dim() == 2 and x.dtype == torch.float32 and x.stride(1) == 1 and w.numel() == x.size(1)
     assert x.size(1) % groups == 0
     out = torch.empty(x.shape, dtype=w.dtype, device=x.device) if out is None else out
+    assert gate is None or (gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.shape == x.shape)
     check(lib().nv_group_rmsnorm_f32(ptr(x), x.stride(0), ptr(w), ptr(out), out.stride(0), x.size(0), groups,
-                                     x.size(1) // groups, eps, _code32(w.dtype), stream()), "nv_group_rmsnorm_f32")
+                                     x.size(1) // groups, eps, ptr(gate), gate.stride(0) if gate is not None else 0,
+                                     _code32(w.dtype), stream()), "nv_group_rmsnorm_f32")
     return out
 
 
@@ -748,6 +811,52 @@ def window_attn(q, cache, block_tables, cu_q, past_lens, seq_of_token, max_q, he
                                ptr(seq_of_token), ptr(out), out.stride(0), T, max_q, heads, kv_heads, dim, vdim,
                                block_size, window, float(softcap or 0.0), out_scale, _code32(cache.dtype), stream()),
           "nv_window_attn")
+    return out
+
+
+def qk_store(proj, offsets, positions, scale, slot_mapping, cache, heads, kv_heads, dim, bias=None, temp_coef=0.0,
+             temp_every=0):
+    """fp32 projections [T, *] with q | k at ``offsets`` (plus ``bias`` over the same columns) -> fp32 queries
+    [T, heads * dim] times ``scale`` and the position temperature 1 + coef * ln(floor((p + 1) / every) + 1) (every 0:
+    none); the keys go to cache rows [G * dim] of ``slot_mapping``: they are the values too."""
+    require_gpu(proj, "qk_store")
+    T = proj.size(0)
+    assert proj.dtype == torch.float32 and proj.stride(1) == 1 and slot_mapping.dtype == torch.int32
+    assert slot_mapping.numel() == T and cache.is_contiguous() and cache.size(-1) == kv_heads * dim
+    assert positions.dtype == torch.int64 and positions.numel() == T and positions.is_contiguous()
+    q_off, k_off = offsets
+    need = max(q_off + heads * dim, k_off + kv_heads * dim)
+    assert need <= proj.size(1)
+    assert bias is None or (bias.dtype == cache.dtype and bias.is_contiguous() and need <= bias.numel() <= proj.size(1))
+    q = torch.empty(T, heads * dim, dtype=torch.float32, device=proj.device)
+    check(lib().nv_qk_store(ptr(proj), ptr(bias), proj.stride(0), q_off, k_off, 0, None, None, None, ptr(positions),
+                            float(temp_coef), int(temp_every), scale, 0.0, ptr(slot_mapping), ptr(cache), ptr(q), T, heads,
+                            kv_heads, dim, 0, _code32(cache.dtype), stream()), "nv_qk_store")
+    return q
+
+
+def paged_softmax_attn(q, cache, block_tables, cu_q, past_lens, seq_of_token, max_q, heads, kv_heads, dim, vdim, block_size,
+                       out, window=0, softcap=0.0, out_scale=1.0, distance_term=False, values_are_keys=False, sink=None,
+                       gate=None):
+    """window_attn with its options spelled out: no distance term unless asked for, cache rows that hold keys only and
+    serve as values too, a sink logit per head in the denominator, a sigmoid gate (fp32 logits laid out like the
+    output) folded into the store."""
+    require_gpu(q, "paged_softmax_attn")
+    T = q.size(0)
+    assert q.dtype == torch.float32 and q.is_contiguous() and q.size(1) == heads * dim and cache.is_contiguous()
+    assert cache.size(-1) == (kv_heads * dim if values_are_keys else kv_heads * (dim + vdim))
+    assert block_tables.dtype == torch.int32 and block_tables.is_contiguous() and block_tables.dim() == 2
+    assert cu_q.dtype == past_lens.dtype == seq_of_token.dtype == torch.int32 and seq_of_token.numel() == T
+    assert out.dtype == cache.dtype and out.stride(1) == 1 and out.size(0) == T and out.size(1) >= heads * vdim
+    assert sink is None or (sink.dtype == cache.dtype and sink.numel() == heads and sink.is_contiguous())
+    assert gate is None or (gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.size(0) == T
+                            and gate.size(1) >= heads * vdim)
+    check(lib().nv_paged_softmax_attn(ptr(q), ptr(cache), ptr(block_tables), block_tables.size(1), ptr(cu_q),
+                                      ptr(past_lens), ptr(seq_of_token), ptr(out), out.stride(0), T, max_q, heads, kv_heads,
+                                      dim, vdim, block_size, window, float(softcap or 0.0), out_scale, int(distance_term),
+                                      int(values_are_keys), ptr(sink), ptr(gate),
+                                      gate.stride(0) if gate is not None else 0, _code32(cache.dtype), stream()),
+          "nv_paged_softmax_attn")
     return out
 
 

@@ -5,7 +5,12 @@ Mixture: fp32 router logits, the ``top`` largest per token, softmax over the cho
 pairs are ordered by expert on the device, the experts' two products run as grouped launches over the gathered rows
 (one weight per group, no host synchronisation: the grid covers the worst case and empty tiles leave at once), and the
 rows are summed per token in the order of its choices.  An optional shared expert runs for every token and is added
-multiplied by sigmoid(w_sg . h), one number per token; its gate row rides in the router's product."""
+multiplied by sigmoid(w_sg . h), one number per token; its gate row rides in the router's product.
+
+Variants a design may choose: ``route="all"`` takes the softmax over every expert and divides the chosen scores by their
+sum (+ 1e-20); the activation ``"clamped"`` is the unit g sigmoid(1.702 g) (u + 1) with g = min(gate, limit) and
+u = clamp(up, -limit, limit); ``forward(h, add)`` folds another fp32 result of the same rows (a mixer that runs beside
+the feed-forward) into the combining launch."""
 
 import torch
 from torch import nn
@@ -13,7 +18,8 @@ from torch import nn
 from byox_vllm_amd import kernels
 from byox_vllm_amd.layers.linear import DenseLinear
 
-ACTIVATIONS = {"silu": kernels.ACT_SILU, "gelu_tanh": kernels.ACT_GELU_TANH}
+ACTIVATIONS = {"silu": kernels.ACT_SILU, "gelu_tanh": kernels.ACT_GELU_TANH, "clamped": kernels.GLU_CLAMPED}
+ROUTES = {"chosen": kernels.ROUTE_CHOSEN, "all": kernels.ROUTE_ALL}
 
 
 class GatedMLP(nn.Module):
@@ -29,9 +35,12 @@ class GatedMLP(nn.Module):
 
 
 class MixtureOfExperts(nn.Module):
-    def __init__(self, width: int, experts: int, top: int, ff: int, act: str = "silu", shared_ff: int | None = None):
+    def __init__(self, width: int, experts: int, top: int, ff: int, act: str = "silu", shared_ff: int | None = None,
+                 route: str = "chosen", limit: float = 0.0):
         super().__init__()
         self.experts, self.top, self.ff, self.width, self.act = experts, top, ff, width, ACTIVATIONS[act]
+        self.route, self.limit = ROUTES[route], float(limit)
+        assert act != "clamped" or self.limit > 0.0
         shards = {"router": experts}
         if shared_ff:
             shards["sg"] = 1
@@ -47,16 +56,17 @@ class MixtureOfExperts(nn.Module):
         at = 0 if part == "gate" else self.ff
         param.data[e, at: at + self.ff].copy_(tensor)
 
-    def forward(self, h):
+    def forward(self, h, add=None):
         T, E, top = h.size(0), self.experts, self.top
         logits = self.router(h, out_dtype=torch.float32)
-        idx, weights = kernels.moe_route(logits, E, top)
+        idx, weights = kernels.moe_route(logits, E, top, self.route)
         offsets, sorted_token, slot_of = kernels.moe_sort(idx, E)
         hidden = kernels.linear(h, self.gate_up.data, rows=T * top, a_rows=sorted_token, batch=E,
                                 w_batch_stride=2 * self.ff * self.width, group_offsets=offsets, max_group_rows=T,
-                                epilogue=kernels.EPI_GLU, act=self.act)
+                                epilogue=kernels.EPI_GLU, act=self.act, cap=self.limit)
         y = kernels.linear(hidden, self.down.data, out_dtype=torch.float32, rows=T * top, batch=E,
                            w_batch_stride=self.width * self.ff, group_offsets=offsets, max_group_rows=T)
         if self.shared is None:
-            return kernels.moe_combine(y, slot_of, weights)
+            return kernels.moe_combine(y, slot_of, weights, add)
+        assert add is None, "a shared expert and an addend share one input of the combining launch"
         return kernels.moe_combine(y, slot_of, weights, self.shared(h), logits[:, E:])

@@ -10,6 +10,7 @@ _MODELS = {
     "Qwen3ForCausalLM": ("byox_vllm_amd.models.qwen3", "Qwen3ForCausalLM"),
     "Rurutar": ("byox_vllm_amd.models.rurutar", "RurutarForCausalLM"),
     "Nonetar": ("byox_vllm_amd.models.nonetar", "NonetarForCausalLM"),
+    "Zamusun": ("byox_vllm_amd.models.zamusun", "ZamusunForCausalLM"),
 }
 DEFAULT = "Qwen3ForCausalLM"
 

@@ -338,7 +338,8 @@ int nv_gemm_lt_f32out(const void* x, int64_t x_row_stride, const void* w_rowmajo
  *   group_offsets  when given, batch b covers the output rows [group_offsets[b], group_offsets[b+1]) (one weight per
  *                expert over rows sorted by expert); M then bounds the rows of one group;
  *   epilogue     0 none; 1 gated unit: W holds N gate rows followed by N up rows, out = act(gate) * up with act = SiLU
- *                (act 0) or the tanh form of GELU (act 1); 2 soft cap: c * tanh(out / c), c = epi_const;
+ *                (act 0) or the tanh form of GELU (act 1), or (act 2) the clamped unit g sigmoid(1.702 g) (u + 1) with
+ *                g = min(gate, c), u = clamp(up, -c, c), c = epi_const; 2 soft cap: c * tanh(out / c), c = epi_const;
  *                3 row gate: out *= sigmoid(epi_ptr[m * epi_row_stride + b]);
  *                4 element-wise function chosen by act: 0 SiLU, 1 tanh-form GELU, 2 xIELU (a z^2 + z/2 for z > 0,
  *                b (exp(z) - 1 - z) + z/2 otherwise, with a = epi_ptr[0], b = epi_ptr[1]), 3 out *= epi_const;
@@ -359,14 +360,20 @@ int nv_embed_scale(const int64_t* ids, const void* table, float* out, int64_t to
 int nv_dyt_norm(float* x, const float* delta, int64_t delta_row_stride, const int32_t* rows_idx, const float* alpha,
                 const void* w, const void* b, void* out, int64_t rows, int n, int dtype, nv_stream_t stream);
 
+/* out[t] = [x[t] | x0[t]] rounded to the storage type, after x += delta in place when delta is given: the input of a
+ * projection that re-enters a block of layers with the first residual beside the current one. */
+int nv_residual_pair(float* x, const float* delta, int64_t delta_row_stride, const float* x0, void* out, int64_t rows,
+                     int n, int dtype, nv_stream_t stream);
+
 /* RMS norm of fp32 rows: out = x / sqrt(mean(x^2) + eps) * w, rounded to the storage type. */
 int nv_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* out, int64_t out_row_stride, int64_t rows,
                    int n, float eps, int dtype, nv_stream_t stream);
 
-/* out[m][j] = act(y[m][j]) * y[m][n + j] over fp32 rows [gate | up] of a plain product; act 0 SiLU, 1 tanh-form GELU. */
+/* out[m][j] = act(y[m][j]) * y[m][n + j] over fp32 rows [gate | up] of a plain product; act as in nv_linear's
+ * epilogue 1, c its limit. */
 /* nv_act_f32: out = f(y) element-wise over fp32 rows of a plain product, f as in nv_linear's epilogue 4. */
 int nv_act_f32(const float* y, void* out, int64_t total, int act, const float* params, float c, int dtype, nv_stream_t stream);
-int nv_act_mul_f32(const float* y, void* out, int64_t rows, int n, int act, int dtype, nv_stream_t stream);
+int nv_act_mul_f32(const float* y, void* out, int64_t rows, int n, int act, float c, int dtype, nv_stream_t stream);
 
 /* Sampler over fp32 logits: temperature 0 -> argmax (lowest index on ties), else Gumbel-max with noise hashed from
  * (seed, row, column). */
@@ -378,6 +385,19 @@ int nv_gla_recurrent(const float* proj, int64_t proj_row_stride, int q_off, int 
                      const float* z, int64_t z_row_stride, float* state, const int32_t* cu_q, const int32_t* past_lens,
                      const int32_t* state_slots, const void* norm_w, void* out, int num_seqs, int heads, int dim,
                      int vdim, float tau, float q_scale, float eps, int dtype, nv_stream_t stream);
+
+/* Matrix memories with one decay per head and token (csrc/memory.hip): S_t = keep_t S_(t-1) + take_t k_t v_t^T,
+ * o_t = S_t^T q_t over this step's tokens of each request, state carried in fp32 slots of nv_matrix_memory_state_size
+ * numbers per head.  mode 0: keep = decay[h], take = 1 (lightning attention); mode 1: exponential gates with a running
+ * maximum and a normaliser (the matrix memory of xLSTM): i = cap tanh(zi / cap), f = logsigmoid(cap tanh(zf / cap)) from
+ * the logits at columns i_off + h and f_off + h of proj (plus `bias`, a vector over proj's columns in the storage type,
+ * may be null), o_t divided by max(|n_t . q_t|, exp(-m_t)) + 1e-6.  silu: q, k and v pass through SiLU first.  out: fp32
+ * rows, head h at columns h * vdim. */
+int64_t nv_matrix_memory_state_size(int mode, int dim, int vdim);
+int nv_matrix_memory(const float* proj, int64_t proj_row_stride, int q_off, int k_off, int v_off, int i_off, int f_off,
+                     const void* bias, const float* decay, float* state, const int32_t* cu_q, const int32_t* past_lens,
+                     const int32_t* state_slots, float* out, int64_t out_row_stride, int num_seqs, int heads, int dim,
+                     int vdim, int mode, int silu, float q_scale, float cap, int dtype, nv_stream_t stream);
 
 /* Latent attention (csrc/latent_attn.hip): cache rows [kv_rank | rot_dim] per token, shared by all heads. */
 int nv_latent_kv_store(const float* kv, int64_t kv_row_stride, const void* norm_w, const int64_t* positions,
@@ -391,9 +411,11 @@ int nv_latent_attn(const float* qa, const void* cache, const int32_t* block_tabl
                    int rank,
                    int rot_dim, int block_size, int window, float scale, int dtype, nv_stream_t stream);
 
-/* Mixture of experts (csrc/moe.hip): routing, ordering by expert, weighted combination. */
+/* Mixture of experts (csrc/moe.hip): routing, ordering by expert, weighted combination.  nv_moe_route mode 0: softmax
+ * over the chosen logits; 1: softmax over all experts, chosen scores divided by (their sum + 1e-20).  nv_moe_combine
+ * adds `shared` times sigmoid(shared_gate) per token, or `shared` as it is when shared_gate is null. */
 int nv_moe_route(const float* logits, int64_t row_stride, int32_t* idx, float* weights, int64_t tokens, int experts,
-                 int top, nv_stream_t stream);
+                 int top, int mode, nv_stream_t stream);
 int nv_moe_sort(const int32_t* idx, int64_t tokens, int experts, int top, int32_t* offsets, int32_t* sorted_token,
                 int32_t* slot_of, nv_stream_t stream);
 int nv_moe_combine(const float* y, const int32_t* slot_of, const float* weights, int top, const float* shared,
@@ -409,7 +431,8 @@ int nv_moe_combine(const float* y, const int32_t* slot_of, const float* weights,
  *   rows_idx gathers rows and leaves the streams as they are.  out is fp32 or the model's type.
  * nv_token_shift: out[t] = h[t] + (h[t-1] - h[t]) * mu; the row before a portion comes from the request's slot of
  *   state [slots, width] (zeros when past_lens is 0), which then receives the portion's last row.
- * nv_group_rmsnorm_f32: fp32 rows of `groups` parts of n numbers, each part divided by its own root mean square. */
+ * nv_group_rmsnorm_f32: fp32 rows of `groups` parts of n numbers, each part divided by its own root mean square, times
+ *   w, times sigmoid(gate) when gate logits (fp32 rows of the same layout) are given. */
 int nv_embed_sinusoid(const int64_t* ids, const int64_t* positions, const void* table, const double* inv_freq, float* out,
                       int64_t tokens, int streams, int width, int64_t vocab, int dtype, nv_stream_t stream);
 int nv_hc_norm(float* x, int streams, int width, const float* delta, int64_t delta_row_stride, const float* hc_prev,
@@ -419,7 +442,8 @@ int nv_token_shift(const float* h, const void* mu, float* state, const int32_t* 
                    const int32_t* state_slots, const int32_t* seq_of_token, void* out, int64_t tokens, int width,
                    int dtype, nv_stream_t stream);
 int nv_group_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* out, int64_t out_row_stride,
-                         int64_t rows, int groups, int n, float eps, int dtype, nv_stream_t stream);
+                         int64_t rows, int groups, int n, float eps, const float* gate, int64_t gate_row_stride,
+                         int dtype, nv_stream_t stream);
 
 /* ---- softmax attention with shaped scores over a paged cache of rows [k: G * dim | v: G * vdim] (csrc/window_attn.hip) ----
  * nv_qk_norm_store: per-head RMS norm of the fp32 q and k projections plus `bias` (a vector over the projection's columns,
@@ -437,6 +461,22 @@ int nv_window_attn(const float* q, const void* cache, const int32_t* block_table
                    const int32_t* past_lens, const int32_t* seq_of_token, void* out, int64_t out_row_stride,
                    int64_t tokens, int max_q, int heads, int kv_heads, int dim, int vdim, int block_size, int window,
                    float softcap, float out_scale, int dtype, nv_stream_t stream);
+/* The general forms.  nv_qk_store: q_norm and k_norm may both be null (no norm), vdim 0 means the values are the keys
+ *   (rows [k: G * dim] only, v_off unused), and with temp_every > 0 the query is also multiplied by
+ *   1 + temp_coef * ln(floor((positions[t] + 1) / temp_every) + 1).
+ * nv_paged_softmax_attn: distance_term 0 drops the distance term; values_are_keys reads rows [k: G * dim] as keys and as
+ *   values (vdim == dim); sink [heads] (storage type, may be null) adds exp(sink[h]) to the softmax's denominator; gate
+ *   (fp32 [tokens, gate_row_stride], head h at h * vdim, may be null) multiplies the output by its sigmoid. */
+int nv_qk_store(const float* proj, const void* bias, int64_t proj_row_stride, int q_off, int k_off, int v_off,
+                const void* q_norm, const void* k_norm, const void* temp, const int64_t* positions, float temp_coef,
+                int temp_every, float scale, float eps, const int32_t* slot_mapping, void* cache, float* q_out,
+                int64_t tokens, int heads, int kv_heads, int dim, int vdim, int dtype, nv_stream_t stream);
+int nv_paged_softmax_attn(const float* q, const void* cache, const int32_t* block_tables, int table_cols,
+                          const int32_t* cu_q, const int32_t* past_lens, const int32_t* seq_of_token, void* out,
+                          int64_t out_row_stride, int64_t tokens, int max_q, int heads, int kv_heads, int dim, int vdim,
+                          int block_size, int window, float softcap, float out_scale, int distance_term,
+                          int values_are_keys, const void* sink, const float* gate, int64_t gate_row_stride, int dtype,
+                          nv_stream_t stream);
 
 /* ---- recurrences with an fp32 state per request (csrc/scan.hip) ----
  * nv_causal_conv: per-channel causal convolution over fp32 rows; state [slots, taps - 1, channels] keeps the last
