@@ -282,7 +282,7 @@ def run_generate_workload(args):
     print(json.dumps(line), flush=True)
 
 
-# --arch-compare: the Rurutar and Nonetar designs beside the dense Qwen3 decoder (and beside each other) at equal
+# --arch-compare: the Rurutar, Nonetar and Zamusun designs beside the dense Qwen3 decoder (and beside each other) at equal
 # width, depth, active feed-forward size and vocabulary, both through LLM.generate: prefill and decode tokens/s.
 # name: (width, layers, prompts, prompt length, decoded tokens)
 ARCH_COMPARE_SIZES = {
@@ -345,13 +345,35 @@ def nonetar_bench_config(width: int, layers: int, vocab: int = 32000):
     return nonetar_config(raw, dtype=torch.bfloat16)
 
 
+def zamusun_bench_config(width: int, layers: int, vocab: int = 32000):
+    """A Zamusun configuration with the proportions of a real model's layers: matrix memories (mLSTM with 64-wide keys
+    and 128-wide values, lightning attention with 128-wide heads) around softmax attention with four query heads per
+    key head of 128; every layer carries a mixture of 16 experts, two per token, whose active size equals the dense
+    comparator's feed-forward.  Two of the layers form a span that runs twice, so ``layers`` counts layer RUNS."""
+    from byox_vllm_amd.models.zamusun import zamusun_config
+    heads = width // 128
+    kinds = [
+        {"type": "mlstm", "mixer": {"heads": heads, "dim": 64, "vdim": 128, "gate_cap": 15.0}},
+        {"type": "lightning", "mixer": {"heads": heads, "dim": 128, "vdim": 128,
+                                        "decay": [1.0 - 2.0 ** -(3 + 5 * h / max(heads - 1, 1)) for h in range(heads)]}},
+        {"type": "attention", "mixer": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128,
+                                        "scale": 128 ** -0.5, "q_temp": {"coef": 0.1, "every": 1024}}},
+    ]
+    moe = {"kind": "moe", "router": {"experts": 16, "top": 2}, "expert": {"ff": 3 * width // 2, "limit": 7.0}}
+    distinct = max(3, layers - 2)
+    specs = [dict(json.loads(json.dumps(kinds[i % 3])), mlp=moe) for i in range(distinct)]
+    raw = {"architecture": "Zamusun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+           "loop": {"start": 2, "stop": 4, "times": 1 + (layers - distinct) // 2}, "layers": specs}
+    return zamusun_config(raw, dtype=torch.bfloat16)
+
+
 def run_arch_compare(args):
     from byox_vllm_amd import LLM, SamplingParams
     from byox_vllm_amd.config import qwen2_config
     assert args.gpus == 1, "--arch-compare runs on one GPU"
     random.seed(0)
     results = []
-    designs = {"rurutar": rurutar_bench_config, "nonetar": nonetar_bench_config}
+    designs = {"rurutar": rurutar_bench_config, "nonetar": nonetar_bench_config, "zamusun": zamusun_bench_config}
     chosen = [d for d in args.arch_designs.split(",") if d]
     assert chosen and all(d in designs for d in chosen), f"--arch-designs: a subset of {sorted(designs)}"
     for name, (width, layers, num, plen, decoded) in ARCH_COMPARE_SIZES.items():
@@ -476,7 +498,7 @@ def main():
                     help="instead of the decode benchmark: prefill and decode tokens/s of the designs named by --arch-designs "
                          "beside the dense Qwen3 decoder at equal size (one GPU, LLM.generate)")
     ap.add_argument("--arch-designs", default="rurutar",
-                    help="--arch-compare: the designs to run beside the dense decoder, comma-separated (rurutar, nonetar)")
+                    help="--arch-compare: the designs to run beside the dense decoder, comma-separated (rurutar, nonetar, zamusun)")
     ap.add_argument("--arch-sizes", default="", help="--arch-compare: comma-separated subset of " + ",".join(ARCH_COMPARE_SIZES))
     args = ap.parse_args()
     if args.arch_compare:

@@ -10,7 +10,8 @@
 // A request's slot holds, per head, S (dim x vdim), then n (dim) and m (1) in the second form.  One workgroup owns one
 // (request, head) pair and walks the request's tokens of this step in order, starting from the slot (or from zero when
 // the request has no tokens behind it) and leaving the state there: a prompt portion, the next portion and single
-// decoded tokens all go through this one kernel.  The results are fp32 rows; the norm and gate that follow them span
+// decoded tokens all go through this one kernel (states that do not fit a workgroup's registers: a slow general kernel
+// that keeps the state in its slot).  The results are fp32 rows; the norm and gate that follow them span
 // heads or not, depending on the design, and run in nv_group_rmsnorm_f32.
 //
 // Thread (cs, v) keeps the entries S[cs * DC .. cs * DC + DC - 1][v] of state column v in registers (the key channels
@@ -188,6 +189,80 @@ __global__ __launch_bounds__(mem_threads(DMAX / CS)) void matrix_memory_kernel(M
   if (MODE == MEM_EXPGATE && tid == 0) n_g[p.dim] = m_run;
 }
 
+// States too large for a workgroup's registers: the state stays in its slot (fp32, through the caches) and is read and
+// written once per token; thread v owns column v, so no two threads touch the same entry.  Slow and general.
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void matrix_memory_generic_kernel(MemArgs p) {
+  extern __shared__ float4 lds4[];
+  float* sk = reinterpret_cast<float*>(lds4);   // [dim]
+  float* sq = sk + p.dim;                       // [dim]
+  float* sg = sq + p.dim;                       // keep, take, exp(-m), then 32 floats for sums
+  float* red = sg + 4;
+  const int vd = p.vdim, tid = threadIdx.x, nthr = blockDim.x;
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int t0 = p.cu_q[b], t1 = p.cu_q[b + 1];
+  if (t1 <= t0) return;
+  float* S_g = p.state + ((int64_t)p.slots[b] * p.H + h) * p.per_head;
+  float* n_g = S_g + (int64_t)p.dim * vd;
+  if (p.past[b] == 0)
+    for (int i = tid; i < p.per_head; i += nthr) S_g[i] = 0.0f;
+  float m_run = (MODE == MEM_EXPGATE && tid == 0 && p.past[b] != 0) ? n_g[p.dim] : 0.0f;
+  const float decay = MODE == MEM_CONST ? p.decay[h] : 0.0f;
+  const T* bias = reinterpret_cast<const T*>(p.bias);
+  __syncthreads();
+  for (int t = t0; t < t1; ++t) {
+    const float* row = p.proj + (int64_t)t * p.proj_rs;
+    for (int i = tid; i < p.dim; i += nthr) {
+      sk[i] = maybe_silu(row[p.k_off + h * p.dim + i], p.silu);
+      sq[i] = maybe_silu(row[p.q_off + h * p.dim + i], p.silu) * p.q_scale;
+    }
+    if (tid == 0) {
+      if constexpr (MODE == MEM_EXPGATE) {
+        float zi = row[p.i_off + h], zf = row[p.f_off + h];
+        if (bias) {
+          zi += ld_f32<T>(bias + p.i_off + h);
+          zf += ld_f32<T>(bias + p.f_off + h);
+        }
+        const float ig = p.cap * tanhf(zi / p.cap);
+        const float fg = log_sigmoid_f32(p.cap * tanhf(zf / p.cap));
+        const float m_new = fmaxf(fg + m_run, ig);
+        sg[0] = expf(fg + m_run - m_new);
+        sg[1] = expf(ig - m_new);
+        sg[2] = expf(-m_new);
+        m_run = m_new;
+      } else {
+        sg[0] = decay;
+        sg[1] = 1.0f;
+        sg[2] = 0.0f;
+      }
+    }
+    __syncthreads();
+    const float keep = sg[0], take = sg[1];
+    float den = 1.0f;
+    if constexpr (MODE == MEM_EXPGATE) {
+      float pn = 0.0f;
+      for (int i = tid; i < p.dim; i += nthr) {
+        const float n = keep * n_g[i] + take * sk[i];
+        n_g[i] = n;
+        pn += n * sq[i];
+      }
+      den = fmaxf(fabsf(block_sum(pn, red)), sg[2]) + 1e-6f;
+    }
+    for (int v = tid; v < vd; v += nthr) {
+      const float vv = maybe_silu(row[p.v_off + h * vd + v], p.silu) * take;
+      float acc = 0.0f;
+      for (int i = 0; i < p.dim; ++i) {
+        const float sv = keep * S_g[(int64_t)i * vd + v] + sk[i] * vv;
+        S_g[(int64_t)i * vd + v] = sv;
+        acc += sv * sq[i];
+      }
+      p.out[(int64_t)t * p.out_rs + h * vd + v] = acc / den;
+    }
+    __syncthreads();   // sk / sq / sg are rewritten by the next token
+  }
+  if (MODE == MEM_EXPGATE && tid == 0) n_g[p.dim] = m_run;
+}
+
 template <typename T, int DMAX, int CS>
 void launch_mem_mode(const MemArgs& p, int mode, dim3 grid, int threads, size_t lds, hipStream_t s) {
   if (mode == MEM_CONST) matrix_memory_kernel<T, DMAX, CS, MEM_CONST><<<grid, dim3(threads), lds, s>>>(p);
@@ -246,15 +321,23 @@ extern "C" int nv_matrix_memory(const float* proj, int64_t proj_row_stride, int 
   int vdp = vround;
   while (vdp * cs < dim) vdp += 64;      // thread d < dim carries n[d]
   const int threads = vdp * cs;
-  if (dmax > 256 || dc > 64 || threads > mem_threads(dc)) {
-    nv_set_error("nv_matrix_memory: a %d x %d state does not fit one workgroup's registers", dim, vdim);
-    return NV_ERR_UNSUPPORTED;
+  MemArgs p{proj, proj_row_stride, q_off, k_off, v_off, i_off, f_off, bias, decay, state, cu_q, past_lens, state_slots,
+            out, out_row_stride, heads, dim, vdim, (int)nv_matrix_memory_state_size(mode, dim, vdim), silu, q_scale, cap};
+  if (dmax > 256 || dc > 64 || threads > mem_threads(dc) || getenv("NV_MATRIX_MEMORY_GENERIC") != nullptr) {
+    const size_t glds = ((size_t)2 * dim + 4 + 32) * sizeof(float);
+    NV_CHECK_ARG(glds <= 64 * 1024, "nv_matrix_memory: keys of %d numbers exceed the LDS", dim);
+    dim3 grid(heads, num_seqs);
+    if (mode == MEM_CONST) {
+      NV_DISPATCH_T(dtype, matrix_memory_generic_kernel<T, MEM_CONST><<<grid, dim3(256), glds, (hipStream_t)stream>>>(p));
+    } else {
+      NV_DISPATCH_T(dtype, matrix_memory_generic_kernel<T, MEM_EXPGATE><<<grid, dim3(256), glds, (hipStream_t)stream>>>(p));
+    }
+    NV_CHECK_LAUNCH();
+    return NV_OK;
   }
   const size_t lds = (size_t)(MM_TC * 2 * dmax + 3 * MM_TC + MM_TC * (threads / 64) + (cs > 1 ? cs * MM_TC * vdp : 0)) *
                      sizeof(float);
   NV_CHECK_ARG(lds <= 64 * 1024, "nv_matrix_memory: %zu bytes of LDS", lds);
-  MemArgs p{proj, proj_row_stride, q_off, k_off, v_off, i_off, f_off, bias, decay, state, cu_q, past_lens, state_slots,
-            out, out_row_stride, heads, dim, vdim, (int)nv_matrix_memory_state_size(mode, dim, vdim), silu, q_scale, cap};
   NV_DISPATCH_T(dtype, launch_mem<T>(p, mode, dmax, cs, dim3(heads, num_seqs), threads, lds, (hipStream_t)stream));
   NV_CHECK_LAUNCH();
   return NV_OK;
