@@ -11,7 +11,8 @@ at 0: keep = exp(f + m_(t-1) - m_t), take = exp(i - m_t); a normaliser n_t follo
 o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6) with q = W_q h / sqrt(dim).  EACH head's o is divided by its own
 root mean square; then weight over all heads, sigmoid(W_g h), projection.
 
-Both read one merged input projection (q | k | v | g [| i | f]) and leave it in fp32: activations, gates, the
+Both read one merged input projection (q | k | v | g [| i | f], then the rows of ``riders``: other consumers of the same
+input, such as a router beside the mixer) and leave it in fp32: activations, gates, the
 recurrence, the norm and the output gate are fp32.  What a request keeps between steps lives in fp32 slots that the
 engine's StateSlotManager hands out; a request's first tokens start from zero instead of reading the slot.  A mixer whose
 layer runs several times per token (a looped span of layers) keeps one state per run: ``runs`` holders, each bound to
@@ -40,14 +41,16 @@ class _MatrixMemoryMixer(nn.Module):
     mode = kernels.MEM_CONST
     extra_shards: tuple = ()
 
-    def __init__(self, width: int, heads: int, dim: int, vdim: int, eps: float, runs: int = 1):
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, eps: float, runs: int = 1, riders: dict | None = None):
         super().__init__()
         self.heads, self.dim, self.vdim, self.eps = heads, dim, vdim, eps
         shards = {"q": heads * dim, "k": heads * dim, "v": heads * vdim, "g": heads * vdim}
         shards.update({name: heads for name in self.extra_shards})
+        shards.update(riders or {})               # rows of other consumers of the same input (a router)
         self.inp = DenseLinear(width, bias=bool(self.extra_shards), shards=shards)
         if self.inp.bias is not None:
             self.inp.bias.data.zero_()            # only the gate rows have a bias; the others keep zero
+            self.inp.bias.keep_init = True        # ... also under random initialisation
         self.at = {name: self.inp.offset(name) for name in shards}
         self.norm = nn.Parameter(torch.ones(heads * vdim), requires_grad=False)
         self.o = DenseLinear(heads * vdim, width)
@@ -62,9 +65,18 @@ class _MatrixMemoryMixer(nn.Module):
 
     norm_groups = 1
 
-    def forward(self, h: torch.Tensor, run: int = 0) -> torch.Tensor:
+    def project(self, h: torch.Tensor) -> torch.Tensor:
+        """The merged input projection, fp32 [T, q | k | v | g | ...]; ``rider(proj, name)`` is a rider's slice of it."""
+        return kernels.linear(h, self.inp.weight.data, out_dtype=torch.float32)
+
+    def rider(self, proj: torch.Tensor, name: str) -> torch.Tensor:
+        at, rows = self.inp.row_of[name]
+        return proj[:, at:at + rows]
+
+    def forward(self, h: torch.Tensor, run: int = 0, positions=None, proj: torch.Tensor | None = None) -> torch.Tensor:
         ctx = get_context()
-        proj = kernels.linear(h, self.inp.weight.data, out_dtype=torch.float32)
+        if proj is None:
+            proj = self.project(h)
         o = self._memory(proj, self.runs[run].state, ctx)
         g = self.at["g"]
         y = kernels.group_rms_norm_f32(o, self.norm.data, self.norm_groups, self.eps,
@@ -75,8 +87,8 @@ class _MatrixMemoryMixer(nn.Module):
 class LightningAttention(_MatrixMemoryMixer):
     mode = kernels.MEM_CONST
 
-    def __init__(self, width: int, heads: int, dim: int, vdim: int, decay, eps: float, runs: int = 1):
-        super().__init__(width, heads, dim, vdim, eps, runs)
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, decay, eps: float, runs: int = 1, riders=None):
+        super().__init__(width, heads, dim, vdim, eps, runs, riders)
         assert len(decay) == heads, f"{len(decay)} decays for {heads} heads"
         self.register_buffer("decay", torch.tensor([float(a) for a in decay], dtype=torch.float32), persistent=False)
 
@@ -90,8 +102,9 @@ class MLSTM(_MatrixMemoryMixer):
     mode = kernels.MEM_EXPGATE
     extra_shards = ("i", "f")
 
-    def __init__(self, width: int, heads: int, dim: int, vdim: int, gate_cap: float, eps: float, runs: int = 1):
-        super().__init__(width, heads, dim, vdim, eps, runs)
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, gate_cap: float, eps: float, runs: int = 1,
+                 riders=None):
+        super().__init__(width, heads, dim, vdim, eps, runs, riders)
         self.gate_cap = float(gate_cap)
         self.norm_groups = heads
 

@@ -10,7 +10,9 @@ multiplied by sigmoid(w_sg . h), one number per token; its gate row rides in the
 Variants a design may choose: ``route="all"`` takes the softmax over every expert and divides the chosen scores by their
 sum (+ 1e-20); the activation ``"clamped"`` is the unit g sigmoid(1.702 g) (u + 1) with g = min(gate, limit) and
 u = clamp(up, -limit, limit); ``forward(h, add)`` folds another fp32 result of the same rows (a mixer that runs beside
-the feed-forward) into the combining launch."""
+the feed-forward) into the combining launch; with ``own_router=False`` the layer has no router matrix and takes fp32
+logits from the caller, whose own projection of the same rows carries the router's rows (one launch and one read of
+the input fewer)."""
 
 import torch
 from torch import nn
@@ -36,7 +38,7 @@ class GatedMLP(nn.Module):
 
 class MixtureOfExperts(nn.Module):
     def __init__(self, width: int, experts: int, top: int, ff: int, act: str = "silu", shared_ff: int | None = None,
-                 route: str = "chosen", limit: float = 0.0):
+                 route: str = "chosen", limit: float = 0.0, own_router: bool = True):
         super().__init__()
         self.experts, self.top, self.ff, self.width, self.act = experts, top, ff, width, ACTIVATIONS[act]
         self.route, self.limit = ROUTES[route], float(limit)
@@ -44,7 +46,8 @@ class MixtureOfExperts(nn.Module):
         shards = {"router": experts}
         if shared_ff:
             shards["sg"] = 1
-        self.router = DenseLinear(width, shards=shards)
+        assert own_router or not shared_ff
+        self.router = DenseLinear(width, shards=shards) if own_router else None
         self.gate_up = nn.Parameter(torch.empty(experts, 2 * ff, width), requires_grad=False)
         self.down = nn.Parameter(torch.empty(experts, width, ff), requires_grad=False)
         self.gate_up.weight_loader = self._load_gate_up
@@ -56,9 +59,11 @@ class MixtureOfExperts(nn.Module):
         at = 0 if part == "gate" else self.ff
         param.data[e, at: at + self.ff].copy_(tensor)
 
-    def forward(self, h, add=None):
+    def forward(self, h, add=None, logits=None):
         T, E, top = h.size(0), self.experts, self.top
-        logits = self.router(h, out_dtype=torch.float32)
+        if logits is None:
+            logits = self.router(h, out_dtype=torch.float32)
+        assert logits.dtype == torch.float32 and logits.shape == (T, E + (1 if self.shared is not None else 0))
         idx, weights = kernels.moe_route(logits, E, top, self.route)
         offsets, sorted_token, slot_of = kernels.moe_sort(idx, E)
         hidden = kernels.linear(h, self.gate_up.data, rows=T * top, a_rows=sorted_token, batch=E,

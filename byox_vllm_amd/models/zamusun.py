@@ -66,31 +66,34 @@ class ZamusunLayer(nn.Module):
         width, eps, m = cfg.hidden_size, cfg.norm_eps, spec["mixer"]
         self.kind = spec["type"]
         self.norm1 = StreamNorm(width, 1, eps, connections=False)
+        mlp = spec.get("mlp")
+        if mlp and mlp["kind"] != "moe":
+            raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+        # mixer and router read the same rows: the router's rows ride in the mixer's input projection
+        riders = {"router": mlp["router"]["experts"]} if mlp else None
         if self.kind == "lightning":
-            self.mix = LightningAttention(width, m["heads"], m["dim"], m["vdim"], m["decay"], eps, runs)
+            self.mix = LightningAttention(width, m["heads"], m["dim"], m["vdim"], m["decay"], eps, runs, riders)
         elif self.kind == "mlstm":
-            self.mix = MLSTM(width, m["heads"], m["dim"], m["vdim"], m["gate_cap"], eps, runs)
+            self.mix = MLSTM(width, m["heads"], m["dim"], m["vdim"], m["gate_cap"], eps, runs, riders)
         elif self.kind == "attention":
             assert m.get("vdim", m["dim"]) == m["dim"], "the values are the keys: they have the keys' size"
             temp = m.get("q_temp") or {}
             self.mix = SinkAttention(width, m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["scale"],
-                                     temp.get("coef", 0.0), temp.get("every", 0), runs)
+                                     temp.get("coef", 0.0), temp.get("every", 0), runs, riders)
         else:
             raise ValueError(f"unknown mixer type {self.kind!r}")
-        mlp = spec.get("mlp")
         self.mlp = None
         if mlp:
-            if mlp["kind"] != "moe":
-                raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
             self.mlp = MixtureOfExperts(width, mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["ff"],
-                                        "clamped", route="all", limit=mlp["expert"]["limit"])
+                                        "clamped", route="all", limit=mlp["expert"]["limit"], own_router=False)
 
     def forward(self, x, delta, positions, run: int):
         """x: fp32 residual [T, width] (updated in place by ``delta``, what the previous layer still owes it) -> what
         this layer owes it: mixer and feed-forward of the same normed rows, summed."""
         h = self.norm1(x.unsqueeze(1), (delta, None) if delta is not None else None)
-        y = self.mix(h, positions, run) if self.kind == "attention" else self.mix(h, run)
-        return self.mlp(h, add=y) if self.mlp is not None else y
+        proj = self.mix.project(h)
+        y = self.mix(h, run, positions, proj)
+        return self.mlp(h, add=y, logits=self.mix.rider(proj, "router")) if self.mlp is not None else y
 
 
 class ZamusunForCausalLM(nn.Module):
@@ -184,7 +187,7 @@ class ZamusunForCausalLM(nn.Module):
             return (base + "mix." + table[leaf][0], table[leaf][1]) if leaf in table else None
         if part == "mlp" and layer.mlp is not None:
             if leaf == "router":
-                return base + "mlp.router.weight", "router"
+                return base + "mix.inp.weight", "router"
             e = self._EXPERT.match(leaf)
             if e and int(e.group(1)) < layer.mlp.experts:
                 if e.group(2) == "down":

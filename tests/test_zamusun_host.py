@@ -107,6 +107,9 @@ def test_every_checkpoint_tensor_has_a_parameter_and_every_parameter_a_tensor(ma
                 assert (mix.inp.bias.data[:mix.at["i"]] == 0).all()
         if layer.mlp is not None:
             e, ff = layer.mlp.experts - 1, layer.mlp.ff
+            at, rows = mix.inp.row_of["router"]                   # the router's rows ride in the mixer's projection
+            assert rows == layer.mlp.experts and at + rows == mix.inp.weight.shape[0] and layer.mlp.router is None
+            assert torch.equal(mix.inp.weight.data[at:], weights[f"l{i}.mlp.router"])
             assert torch.equal(layer.mlp.gate_up.data[e, ff:], weights[f"l{i}.mlp.e{e}.up"])
             assert torch.equal(layer.mlp.down.data[0], weights[f"l{i}.mlp.e0.down"])
 
