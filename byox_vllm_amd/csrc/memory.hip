@@ -7,14 +7,16 @@
 //              from one logit each per head, a running maximum m_t = max(f_t + m_(t-1), i_t) that starts at 0,
 //              keep_t = exp(f_t + m_(t-1) - m_t), take_t = exp(i_t - m_t); a normaliser n_t = keep_t n_(t-1) + take_t k_t
 //              runs beside S, and o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6).
-// A request's slot holds, per head, S (dim x vdim), then n (dim) and m (1) in the second form.  One workgroup owns one
-// (request, head) pair and walks the request's tokens of this step in order, starting from the slot (or from zero when
+// A request's slot holds, per head, S (dim x vdim), then in the second form n (dim) and m (1) once per slice of 64 value
+// columns.  One workgroup owns one (request, head, slice of 64 state columns) triple - columns are independent of each
+// other, so slices need nothing from each other but each keeps its own copy of the normaliser and the maximum; launches
+// of many requests give a workgroup all slices of a head instead - and walks the request's tokens of this step in order, starting from the slot (or from zero when
 // the request has no tokens behind it) and leaving the state there: a prompt portion, the next portion and single
 // decoded tokens all go through this one kernel (states that do not fit a workgroup's registers: a slow general kernel
 // that keeps the state in its slot).  The results are fp32 rows; the norm and gate that follow them span
 // heads or not, depending on the design, and run in nv_group_rmsnorm_f32.
 //
-// Thread (cs, v) keeps the entries S[cs * DC .. cs * DC + DC - 1][v] of state column v in registers (the key channels
+// Thread (cs, v) keeps the entries S[cs * DC .. cs * DC + DC - 1][v] of state column v of its slice in registers (the key channels
 // of a column are split over CS threads; their partial o_t meet in LDS once per chunk of tokens).  Tokens are staged
 // sixteen at a time: k and q rows in LDS (padded to DMAX with zeros), the thread's own v values in registers; the gates
 // of the chunk are a scalar recurrence that one thread walks while the others stage.  Thread d < dim also carries n[d];
@@ -44,14 +46,15 @@ struct MemArgs {
 
 __device__ __forceinline__ float maybe_silu(float z, int on) { return on ? silu_f32(z) : z; }
 
-constexpr int mem_threads(int per_thread) { return per_thread >= 64 ? 256 : 512; }   // by state registers per thread
+constexpr int MEM_SLICE = 64;      // state columns that share one copy of n | m
 
 template <typename T, int DMAX, int CS, int MODE>
-__global__ __launch_bounds__(mem_threads(DMAX / CS)) void matrix_memory_kernel(MemArgs p) {
+__global__ __launch_bounds__(256) void matrix_memory_kernel(MemArgs p) {
   constexpr int DC = DMAX / CS;
   extern __shared__ float4 lds4[];
   float* lds = reinterpret_cast<float*>(lds4);
   const int vd = p.vdim;
+  // the workgroup covers vdp state columns (a multiple of 64: one slice, or several when the launch has workgroups enough)
   const int tid = threadIdx.x, nthr = blockDim.x, vdp = nthr / CS, nwt = nthr >> 6;
   float* sk = lds;                       // [TC][DMAX]
   float* sq = sk + MM_TC * DMAX;         // [TC][DMAX]
@@ -59,14 +62,17 @@ __global__ __launch_bounds__(mem_threads(DMAX / CS)) void matrix_memory_kernel(M
   float* sred = sg + 3 * MM_TC;          // [TC][wavefronts] partial n . q
   float* so = sred + MM_TC * nwt;        // [CS][TC][vdp] partial outputs (CS > 1)
   const int h = blockIdx.x, b = blockIdx.y;
-  const int v = tid % vdp, cs = tid / vdp;
+  const int vl = tid % vdp, cs = tid / vdp;          // column inside the slice, split of the key channels
+  const int v = blockIdx.z * vdp + vl;
   const int cb = cs * DC;
   const bool active = v < vd;
   const int col = active ? v : 0;
   const int t0 = p.cu_q[b], t1 = p.cu_q[b + 1];
   if (t1 <= t0) return;
   float* S_g = p.state + ((int64_t)p.slots[b] * p.H + h) * p.per_head;
-  float* n_g = S_g + (int64_t)p.dim * vd;
+  const int copy0 = blockIdx.z * (vdp / MEM_SLICE);                     // first of the n | m copies this workgroup owns
+  const int ncopies = min(vdp / MEM_SLICE, (vd + MEM_SLICE - 1) / MEM_SLICE - copy0);
+  float* n_g = S_g + (int64_t)p.dim * vd + (int64_t)copy0 * (p.dim + 1);
   const bool fresh = p.past[b] == 0;
   float S[DC];
 #pragma unroll
@@ -150,7 +156,7 @@ __global__ __launch_bounds__(mem_threads(DMAX / CS)) void matrix_memory_kernel(M
     }
     if constexpr (CS > 1) {
 #pragma unroll
-      for (int j = 0; j < MM_TC; ++j) so[(cs * MM_TC + j) * vdp + v] = o[j];
+      for (int j = 0; j < MM_TC; ++j) so[(cs * MM_TC + j) * vdp + vl] = o[j];
     }
     if constexpr (MODE == MEM_EXPGATE) {
 #pragma unroll
@@ -168,7 +174,7 @@ __global__ __launch_bounds__(mem_threads(DMAX / CS)) void matrix_memory_kernel(M
           if constexpr (CS > 1) {
             r = 0.0f;
 #pragma unroll
-            for (int q = 0; q < CS; ++q) r += so[(q * MM_TC + j) * vdp + v];
+            for (int q = 0; q < CS; ++q) r += so[(q * MM_TC + j) * vdp + vl];
           }
           if constexpr (MODE == MEM_EXPGATE) {
             float nq = 0.0f;
@@ -185,8 +191,10 @@ __global__ __launch_bounds__(mem_threads(DMAX / CS)) void matrix_memory_kernel(M
     for (int i = 0; i < DC; ++i)
       if (cb + i < p.dim) S_g[(int64_t)(cb + i) * vd + v] = S[i];
   }
-  if (has_n) n_g[tid] = nreg;
-  if (MODE == MEM_EXPGATE && tid == 0) n_g[p.dim] = m_run;
+  for (int c = 0; c < ncopies; ++c) {
+    if (has_n) n_g[c * (p.dim + 1) + tid] = nreg;
+    if (MODE == MEM_EXPGATE && tid == 0) n_g[c * (p.dim + 1) + p.dim] = m_run;
+  }
 }
 
 // States too large for a workgroup's registers: the state stays in its slot (fp32, through the caches) and is read and
@@ -203,7 +211,8 @@ __global__ __launch_bounds__(256) void matrix_memory_generic_kernel(MemArgs p) {
   const int t0 = p.cu_q[b], t1 = p.cu_q[b + 1];
   if (t1 <= t0) return;
   float* S_g = p.state + ((int64_t)p.slots[b] * p.H + h) * p.per_head;
-  float* n_g = S_g + (int64_t)p.dim * vd;
+  float* n_g = S_g + (int64_t)p.dim * vd;           // copies of n | m, one per 64 value columns, all kept equal
+  const int copies = (vd + MEM_SLICE - 1) / MEM_SLICE;
   if (p.past[b] == 0)
     for (int i = tid; i < p.per_head; i += nthr) S_g[i] = 0.0f;
   float m_run = (MODE == MEM_EXPGATE && tid == 0 && p.past[b] != 0) ? n_g[p.dim] : 0.0f;
@@ -243,7 +252,7 @@ __global__ __launch_bounds__(256) void matrix_memory_generic_kernel(MemArgs p) {
       float pn = 0.0f;
       for (int i = tid; i < p.dim; i += nthr) {
         const float n = keep * n_g[i] + take * sk[i];
-        n_g[i] = n;
+        for (int c = 0; c < copies; ++c) n_g[c * (p.dim + 1) + i] = n;
         pn += n * sq[i];
       }
       den = fmaxf(fabsf(block_sum(pn, red)), sg[2]) + 1e-6f;
@@ -260,7 +269,8 @@ __global__ __launch_bounds__(256) void matrix_memory_generic_kernel(MemArgs p) {
     }
     __syncthreads();   // sk / sq / sg are rewritten by the next token
   }
-  if (MODE == MEM_EXPGATE && tid == 0) n_g[p.dim] = m_run;
+  if (MODE == MEM_EXPGATE && tid == 0)
+    for (int c = 0; c < copies; ++c) n_g[c * (p.dim + 1) + p.dim] = m_run;
 }
 
 template <typename T, int DMAX, int CS>
@@ -294,7 +304,7 @@ void launch_mem(const MemArgs& p, int mode, int dmax, int cs, dim3 grid, int thr
 }  // namespace
 
 extern "C" int64_t nv_matrix_memory_state_size(int mode, int dim, int vdim) {
-  return (int64_t)dim * vdim + (mode == MEM_EXPGATE ? dim + 1 : 0);
+  return (int64_t)dim * vdim + (mode == MEM_EXPGATE ? (int64_t)((vdim + MEM_SLICE - 1) / MEM_SLICE) * (dim + 1) : 0);
 }
 
 extern "C" int nv_matrix_memory(const float* proj, int64_t proj_row_stride, int q_off, int k_off, int v_off, int i_off,
@@ -312,18 +322,25 @@ extern "C" int nv_matrix_memory(const float* proj, int64_t proj_row_stride, int 
   if (num_seqs == 0) return NV_OK;
   int dmax = 16;
   while (dmax < dim) dmax *= 2;
-  const int vround = ((vdim + 63) / 64) * 64;
-  // split a column's key channels over more threads while the workgroup stays within 256 threads, and as far as needed
-  // to keep a thread's part of the column within 64 registers
-  int cs = 1;
-  while (cs < 4 && dmax / (cs * 2) >= 16 && (vround * cs * 2 <= 256 || dmax / cs > 64)) cs *= 2;
-  const int dc = dmax / cs;
-  int vdp = vround;
-  while (vdp * cs < dim) vdp += 64;      // thread d < dim carries n[d]
+  // One workgroup per slice of 64 state columns, the key channels of a column split over as many threads as leave each
+  // at least 16 of them ...
+  int slices = (vdim + MEM_SLICE - 1) / MEM_SLICE, cs = dmax >= 64 ? 4 : dmax / 16, vdp = MEM_SLICE;
+  // ... unless the launch fills the chip anyway (many requests): then one workgroup walks all columns, if that fits 256
+  // threads with at most 64 state registers each (shared staging and fewer, fuller workgroups win there)
+  if (slices > 1 && (int64_t)heads * num_seqs >= 512) {
+    const int vround = slices * MEM_SLICE;
+    int cu = 1;
+    while (cu < 4 && vround * cu * 2 <= 256 && dmax / (cu * 2) >= 16) cu *= 2;
+    if (vround * cu <= 256 && dmax / cu <= 64 && vround * cu >= dim) {
+      cs = cu;
+      vdp = vround;
+      slices = 1;
+    }
+  }
   const int threads = vdp * cs;
   MemArgs p{proj, proj_row_stride, q_off, k_off, v_off, i_off, f_off, bias, decay, state, cu_q, past_lens, state_slots,
             out, out_row_stride, heads, dim, vdim, (int)nv_matrix_memory_state_size(mode, dim, vdim), silu, q_scale, cap};
-  if (dmax > 256 || dc > 64 || threads > mem_threads(dc) || getenv("NV_MATRIX_MEMORY_GENERIC") != nullptr) {
+  if (dmax > 256 || slices > 65535 || getenv("NV_MATRIX_MEMORY_GENERIC") != nullptr) {
     const size_t glds = ((size_t)2 * dim + 4 + 32) * sizeof(float);
     NV_CHECK_ARG(glds <= 64 * 1024, "nv_matrix_memory: keys of %d numbers exceed the LDS", dim);
     dim3 grid(heads, num_seqs);
@@ -335,10 +352,10 @@ extern "C" int nv_matrix_memory(const float* proj, int64_t proj_row_stride, int 
     NV_CHECK_LAUNCH();
     return NV_OK;
   }
-  const size_t lds = (size_t)(MM_TC * 2 * dmax + 3 * MM_TC + MM_TC * (threads / 64) + (cs > 1 ? cs * MM_TC * vdp : 0)) *
-                     sizeof(float);
-  NV_CHECK_ARG(lds <= 64 * 1024, "nv_matrix_memory: %zu bytes of LDS", lds);
-  NV_DISPATCH_T(dtype, launch_mem<T>(p, mode, dmax, cs, dim3(heads, num_seqs), threads, lds, (hipStream_t)stream));
+  const size_t lds =
+      (size_t)(MM_TC * 2 * dmax + 3 * MM_TC + MM_TC * (threads / 64) + (cs > 1 ? cs * MM_TC * vdp : 0)) * sizeof(float);
+  NV_CHECK_ARG(lds <= 64 * 1024 && threads <= 256, "nv_matrix_memory: launch plan out of range");
+  NV_DISPATCH_T(dtype, launch_mem<T>(p, mode, dmax, cs, dim3(heads, num_seqs, slices), threads, lds, (hipStream_t)stream));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

@@ -583,8 +583,9 @@ MEM_CONST, MEM_EXPGATE = 0, 1
 
 
 def matrix_memory_state_size(mode, dim, vdim) -> int:
-    """fp32 numbers one head keeps between steps: the matrix, and in the gated form the normaliser and the maximum."""
-    return dim * vdim + (dim + 1 if mode == MEM_EXPGATE else 0)
+    """fp32 numbers one head keeps between steps: the matrix, and in the gated form the normaliser and the maximum, once
+    per slice of 64 value columns (each slice is walked by a workgroup of its own).  Mirrors nv_matrix_memory_state_size."""
+    return dim * vdim + (-(-vdim // 64) * (dim + 1) if mode == MEM_EXPGATE else 0)
 
 
 def matrix_memory(proj, offsets, state, cu_q, past_lens, state_slots, heads, dim, vdim, mode, *, decay=None, bias=None,

@@ -388,7 +388,7 @@ int nv_gla_recurrent(const float* proj, int64_t proj_row_stride, int q_off, int 
 
 /* Matrix memories with one decay per head and token (csrc/memory.hip): S_t = keep_t S_(t-1) + take_t k_t v_t^T,
  * o_t = S_t^T q_t over this step's tokens of each request, state carried in fp32 slots of nv_matrix_memory_state_size
- * numbers per head.  mode 0: keep = decay[h], take = 1 (lightning attention); mode 1: exponential gates with a running
+ * numbers per head (the matrix; in mode 1 also normaliser and maximum, one copy per 64 value columns).  mode 0: keep = decay[h], take = 1 (lightning attention); mode 1: exponential gates with a running
  * maximum and a normaliser (the matrix memory of xLSTM): i = cap tanh(zi / cap), f = logsigmoid(cap tanh(zf / cap)) from
  * the logits at columns i_off + h and f_off + h of proj (plus `bias`, a vector over proj's columns in the storage type,
  * may be null), o_t divided by max(|n_t . q_t|, exp(-m_t)) + 1e-6.  silu: q, k and v pass through SiLU first.  out: fp32

@@ -77,7 +77,7 @@ def _memory_run(proj, offs, goffs, pieces, H, d, dv, mode, state, slot=0, decay=
     return torch.cat(outs)
 
 
-# the last three do not fit a workgroup's registers and take the general kernel
+# value sizes above 64 are walked in slices of 64 columns by workgroups of their own; keys above 256 take the general kernel
 SHAPES = [(3, 16, 24), (1, 12, 20), (2, 64, 64), (1, 128, 128), (2, 128, 32), (1, 256, 40), (5, 8, 130), (2, 40, 8),
           (1, 300, 20), (2, 256, 128), (1, 130, 300)]
 
@@ -97,6 +97,66 @@ def test_matrix_memory_in_pieces(mode, H, d, dv, pieces):
     want = _memory_plain(proj, offs, goffs, H, d, dv, mode, decay=decay, bias=bias, cap=7.0)
     _close(got, want, 2e-5)
     assert torch.isnan(state[0]).all() and torch.isnan(state[2]).all() and not torch.isnan(state[1]).any()
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("H,d,dv", [(2, 24, 16), (1, 64, 130)])
+def test_matrix_memory_general_kernel_shares_the_slot_layout(mode, H, d, dv, monkeypatch):
+    """The general kernel continues a state the fast kernel left, and the other way round."""
+    from byox_vllm_amd import kernels
+    assert kernels.matrix_memory_state_size(mode, d, dv) == kernels.lib().nv_matrix_memory_state_size(mode, d, dv)
+    proj, offs, goffs = _memory_inputs(45, H, d, dv, seed=9)
+    decay, bias = [0.9] * H, (torch.zeros(H), torch.ones(H))
+    want = _memory_plain(proj, offs, goffs, H, d, dv, mode, decay=decay, bias=bias, cap=9.0)
+    for first_general in (True, False):
+        state = torch.full((1, H, kernels.matrix_memory_state_size(mode, d, dv)), float("nan"), device=DEV)
+        outs = []
+        for k, (a, b) in enumerate(((0, 20), (20, 21), (21, 45))):
+            if (k % 2 == 0) == first_general:
+                monkeypatch.setenv("NV_MATRIX_MEMORY_GENERIC", "1")
+            else:
+                monkeypatch.delenv("NV_MATRIX_MEMORY_GENERIC", raising=False)
+            outs.append(_memory_run(proj[a:b], offs, goffs, [b - a], H, d, dv, mode, state, decay=decay, bias=bias, cap=9.0)
+                        if a == 0 else _memory_continue(proj[a:b], offs, goffs, a, H, d, dv, mode, state, decay, bias, 9.0))
+        monkeypatch.delenv("NV_MATRIX_MEMORY_GENERIC", raising=False)
+        _close(torch.cat(outs), want, 2e-5)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_matrix_memory_many_requests_take_whole_heads_and_few_take_slices(mode):
+    """64 requests x 8 heads give one workgroup all 128 value columns of a head; the two requests that go on alone are
+    then walked in slices of 64 columns, from the state the first launch left."""
+    from byox_vllm_amd import kernels
+    H, d, dv, B = 8, 16, 128, 64
+    projs = [_memory_inputs(5, H, d, dv, seed=200 + i) for i in range(B)]
+    offs, goffs = projs[0][1], projs[0][2]
+    decay, bias = [0.8 + 0.02 * h for h in range(H)], (torch.zeros(H), torch.ones(H))
+    state = torch.full((B, H, kernels.matrix_memory_state_size(mode, d, dv)), float("nan"), device=DEV)
+    bias_full = torch.zeros(projs[0][0].shape[1], device=DEV)
+    bias_full[goffs[1]:goffs[1] + H] = 1.0
+    kw = dict(decay=torch.tensor(decay, device=DEV), bias=bias_full if mode else None, gate_offsets=goffs, cap=5.0,
+              silu=mode == 0, q_scale=d ** -0.5 if mode else 1.0)
+    batch = torch.cat([p[0][:3] for p in projs]).to(DEV)
+    got1 = kernels.matrix_memory(batch, offs, state, _i32(list(range(0, 3 * B + 1, 3))), _i32([0] * B), _i32(list(range(B))),
+                                 H, d, dv, mode, **kw)
+    keep = [7, 50]
+    batch = torch.cat([projs[r][0][3:] for r in keep]).to(DEV)
+    got2 = kernels.matrix_memory(batch, offs, state, _i32([0, 2, 4]), _i32([3, 3]), _i32(keep), H, d, dv, mode, **kw)
+    for k, r in enumerate(keep):
+        want = _memory_plain(projs[r][0], offs, goffs, H, d, dv, mode, decay=decay, bias=bias, cap=5.0)
+        _close(torch.cat([got1[3 * r:3 * r + 3], got2[2 * k:2 * k + 2]]), want, 2e-5)
+    want = _memory_plain(projs[33][0][:3], offs, goffs, H, d, dv, mode, decay=decay, bias=bias, cap=5.0)
+    _close(got1[99:102], want, 2e-5)
+
+
+def _memory_continue(proj, offs, goffs, past, H, d, dv, mode, state, decay, bias, cap):
+    from byox_vllm_amd import kernels
+    n = proj.shape[0]
+    bias_full = torch.zeros(proj.shape[1], device=DEV)
+    bias_full[goffs[0]:goffs[0] + H], bias_full[goffs[1]:goffs[1] + H] = bias[0].to(DEV), bias[1].to(DEV)
+    return kernels.matrix_memory(proj.to(DEV), offs, state, _i32([0, n]), _i32([past]), _i32([0]), H, d, dv, mode,
+                                 decay=torch.tensor(decay, device=DEV), bias=bias_full if mode else None,
+                                 gate_offsets=goffs, cap=cap, silu=mode == 0, q_scale=d ** -0.5 if mode else 1.0)
 
 
 @pytest.mark.parametrize("mode", [0, 1])

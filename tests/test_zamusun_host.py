@@ -64,6 +64,8 @@ def test_every_run_of_a_looped_layer_has_its_own_cache_and_state():
     # mlstm: matrix + normaliser + maximum per head; lightning: the matrix alone, once per run
     assert [r.state_spec()["shape"] for r in m.state_layers()] == [(3, 16 * 24 + 16 + 1), (2, 24 * 16), (2, 24 * 16),
                                                                     (2, 8 * 40 + 8 + 1)]
+    w = ZamusunForCausalLM(zamusun_config(wide_config(), dtype=torch.float32))      # 128 value columns: two slices
+    assert w.state_layers()[0].state_spec()["shape"] == (1, 128 * 128 + 2 * (128 + 1))
     assert len({id(r) for r in m.page_layers() + m.state_layers()}) == 6
     p = ZamusunForCausalLM(zamusun_config(plain_config(), dtype=torch.float32))
     assert p.loop_in is None and len(p.page_layers()) == 1 and len(p.state_layers()) == 1
