@@ -93,7 +93,8 @@ _PROTOS = {
     "nv_window_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _p]),
     "nv_qk_store": (_i, [_p, _p, _i64, _i, _i, _i, _p, _p, _p, _p, _f, _i, _f, _f, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _p]),
     "nv_paged_softmax_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
-                                   _p, _p, _i64, _i, _p]),
+                                   _p, _p, _i64, _p, _sz, _i, _p]),
+    "nv_paged_softmax_attn_workspace_bytes": (_sz, [_i64, _i, _i, _i, _i]),
     "nv_causal_conv": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _i, _i, _i, _i, _p]),
     "nv_rglru_scan": (_i, [_p, _i64, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _i, _f, _f, _i, _p]),
     "nv_ssd_scan": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _sz, _i,

@@ -160,6 +160,38 @@ __global__ __launch_bounds__(256) void group_rmsnorm_f32_kernel(const float* __r
   }
 }
 
+// the same for parts of at most 256 numbers: one wavefront per part, four parts per workgroup, no LDS
+template <typename T>
+__global__ __launch_bounds__(256) void group_rmsnorm_f32_wave_kernel(const float* __restrict__ x, int64_t x_rs,
+                                                                     const T* __restrict__ w, T* __restrict__ out,
+                                                                     int64_t out_rs, int64_t parts, int groups, int n,
+                                                                     float eps, const float* __restrict__ gate,
+                                                                     int64_t gate_rs) {
+  const int64_t part = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (part >= parts) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = part / groups;
+  const int g = (int)(part % groups);
+  const float* xr = x + t * x_rs + (int64_t)g * n;
+  float v[4], ss = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int j = lane + 64 * i;
+    v[i] = j < n ? xr[j] : 0.0f;
+    ss += v[i] * v[i];
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int j = lane + 64 * i;
+    if (j >= n) continue;
+    float y = v[i] * inv * ld_f32<T>(w + (int64_t)g * n + j);
+    if (gate) y *= sigmoid_f32(gate[t * gate_rs + (int64_t)g * n + j]);
+    st_f32<T>(out + t * out_rs + (int64_t)g * n + j, y);
+  }
+}
+
 }  // namespace
 
 extern "C" int nv_embed_sinusoid(const int64_t* ids, const int64_t* positions, const void* table, const double* inv_freq,
@@ -224,6 +256,15 @@ extern "C" int nv_group_rmsnorm_f32(const float* x, int64_t x_row_stride, const 
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_group_rmsnorm_f32: bad dtype %d", dtype);
   NV_CHECK_ARG(rows >= 0 && n > 0 && groups > 0 && rows * groups < (1ll << 31), "nv_group_rmsnorm_f32: bad shape");
   if (rows == 0) return NV_OK;
+  if (n <= 256 && groups > 1) {
+    const int64_t parts = rows * groups;
+    NV_DISPATCH_T(dtype, group_rmsnorm_f32_wave_kernel<T><<<dim3((unsigned)((parts + 3) / 4)), dim3(256), 0,
+                                                            (hipStream_t)stream>>>(
+                             x, x_row_stride, (const T*)w, (T*)out, out_row_stride, parts, groups, n, eps, gate,
+                             gate_row_stride));
+    NV_CHECK_LAUNCH();
+    return NV_OK;
+  }
   NV_DISPATCH_T(dtype, group_rmsnorm_f32_kernel<T><<<dim3((unsigned)(rows * groups)), dim3(256), 0, (hipStream_t)stream>>>(
                            x, x_row_stride, (const T*)w, (T*)out, out_row_stride, groups, n, eps, gate, gate_row_stride));
   NV_CHECK_LAUNCH();

@@ -101,6 +101,8 @@ struct WAttnArgs {
   const void* sink;        // [H] logits that join the denominator, or null
   const float* gate;       // [tokens, gate_rs] logits whose sigmoid multiplies the output (head h at h * dv), or null
   int64_t gate_rs;
+  int ksplit;              // SPLIT only: workgroups that share a token's keys (blockIdx.z); > 1: results go to `partial`
+  float* partial;          // [tokens, H, ksplit, dv + 2]: unnormalised output, then maximum and sum
 };
 
 // (factor for the accumulated values, denominator) once the walk over the keys is over: the sink joins the sum
@@ -320,7 +322,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
     const int wpos_lo = p0 + row0 / R, wpos_hi = p0 + min(rows - 1, row0 + 15) / R;
 
     const int lo = p.window > 0 ? max(0, p0 - p.window + 1) : 0, hi = p0 + nq - 1;
-    for (int j0 = lo + (SPLIT ? wv * MA_KEYS : 0); j0 <= hi; j0 += SPLIT ? 4 * MA_KEYS : MA_KEYS) {
+    const int walkers = SPLIT ? 4 * p.ksplit : 1;          // wavefronts (of all workgroups) that share this token's keys
+    for (int j0 = lo + (SPLIT ? ((int)blockIdx.z * 4 + wv) * MA_KEYS : 0); j0 <= hi; j0 += walkers * MA_KEYS) {
       if (stid < MA_KEYS) {
         const int kp = j0 + stid;
         sRow[stid] = kp <= hi ? (int64_t)table[kp / p.block_size] * p.block_size + kp % p.block_size : -1;
@@ -457,6 +460,15 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
           o += pw[rr * PW + e] * f;
         }
         const int h = g * R + rr % R;
+        if (p.ksplit > 1) {      // another launch joins the workgroups' shares (and the sink, and the gate)
+          float* dst = p.partial + (((ts + rr / R) * p.H + h) * p.ksplit + blockIdx.z) * (dv + 2);
+          dst[e] = o;
+          if (e == 0) {
+            dst[dv] = m;
+            dst[dv + 1] = l;
+          }
+          continue;
+        }
         float f, den;
         close_softmax(m, l, sink != nullptr, sink ? ld_f32<bf16_t>(sink + h) : 0.0f, f, den);
         float v = o * f * p.out_scale / den;
@@ -483,6 +495,36 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
       }
     }
     ts = te;
+  }
+}
+
+// joins the shares of the ksplit workgroups that walked one token's keys: one wavefront per (token, head)
+__global__ __launch_bounds__(256) void window_attn_join_kernel(WAttnArgs p) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= p.tokens * p.H) return;
+  const int lane = threadIdx.x & 63, dv = p.dv, h = (int)(row % p.H);
+  const int64_t t = row / p.H;
+  const float* src = p.partial + row * p.ksplit * (dv + 2);
+  float m = -INFINITY;
+  for (int z = 0; z < p.ksplit; ++z) m = fmaxf(m, src[z * (dv + 2) + dv]);
+  float l = 0.0f;
+  for (int z = 0; z < p.ksplit; ++z) {
+    const float mz = src[z * (dv + 2) + dv];
+    l += mz == -INFINITY ? 0.0f : src[z * (dv + 2) + dv + 1] * __expf(mz - m);
+  }
+  const bf16_t* sink = reinterpret_cast<const bf16_t*>(p.sink);
+  float f, den;
+  close_softmax(m, l, sink != nullptr, sink ? ld_f32<bf16_t>(sink + h) : 0.0f, f, den);
+  bf16_t* out = reinterpret_cast<bf16_t*>(p.out) + t * p.out_rs + h * dv;
+  for (int e = lane; e < dv; e += 64) {
+    float o = 0.0f;
+    for (int z = 0; z < p.ksplit; ++z) {
+      const float mz = src[z * (dv + 2) + dv];
+      o += mz == -INFINITY ? 0.0f : src[z * (dv + 2) + e] * __expf(mz - m);
+    }
+    float v = o * f * p.out_scale / den;
+    if (p.gate) v *= sigmoid_f32(p.gate[t * p.gate_rs + h * dv + e]);
+    out[e] = (bf16_t)v;
   }
 }
 
@@ -520,6 +562,21 @@ hipError_t launch_window_mfma(const WAttnArgs& p, int ct, bool split, dim3 grid,
 
 }  // namespace
 
+// Workgroups that share one decoded token's keys: enough to put about 256 workgroups on the chip, at most 8.  A
+// function of the launch shape alone (not of the contexts), so a captured launch stays valid as contexts grow.
+static int window_attn_key_splits(int64_t tokens, int kv_heads) {
+  const int64_t groups = tokens * kv_heads;
+  int k = 1;
+  while (k < 8 && groups * k * 2 <= 256) k *= 2;
+  return k;
+}
+
+extern "C" size_t nv_paged_softmax_attn_workspace_bytes(int64_t tokens, int max_q, int heads, int kv_heads, int vdim) {
+  if (max_q > 1 || tokens <= 0 || heads / kv_heads > 16) return 0;
+  const int k = window_attn_key_splits(tokens, kv_heads);
+  return k > 1 ? (size_t)tokens * heads * k * (vdim + 2) * sizeof(float) : 0;
+}
+
 extern "C" int nv_qk_store(const float* proj, const void* bias, int64_t proj_row_stride, int q_off, int k_off, int v_off,
                            const void* q_norm, const void* k_norm, const void* temp, const int64_t* positions,
                            float temp_coef, int temp_every, float scale, float eps, const int32_t* slot_mapping,
@@ -554,7 +611,7 @@ extern "C" int nv_window_attn(const float* q, const void* cache, const int32_t* 
                               int block_size, int window, float softcap, float out_scale, int dtype, nv_stream_t stream) {
   return nv_paged_softmax_attn(q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride,
                                tokens, max_q, heads, kv_heads, dim, vdim, block_size, window, softcap, out_scale, 1, 0,
-                               nullptr, nullptr, 0, dtype, stream);
+                               nullptr, nullptr, 0, nullptr, 0, dtype, stream);
 }
 
 extern "C" int nv_paged_softmax_attn(const float* q, const void* cache, const int32_t* block_tables, int table_cols,
@@ -562,7 +619,7 @@ extern "C" int nv_paged_softmax_attn(const float* q, const void* cache, const in
                                      int64_t out_row_stride, int64_t tokens, int max_q, int heads, int kv_heads, int dim,
                                      int vdim, int block_size, int window, float softcap, float out_scale, int distance_term,
                                      int values_are_keys, const void* sink, const float* gate, int64_t gate_row_stride,
-                                     int dtype, nv_stream_t stream) {
+                                     void* workspace, size_t workspace_bytes, int dtype, nv_stream_t stream) {
   NV_CHECK_ARG(q && cache && block_tables && cu_q && past_lens && seq_of_token && out, "nv_window_attn: null pointer");
   NV_CHECK_ARG(!values_are_keys || vdim == dim, "nv_window_attn: values that are the keys have the keys' size");
   const int cw = values_are_keys ? kv_heads * dim : kv_heads * (dim + vdim), v_col = values_are_keys ? 0 : kv_heads * dim;
@@ -578,12 +635,17 @@ extern "C" int nv_paged_softmax_attn(const float* q, const void* cache, const in
     const int ks = dim <= 64 ? 2 : dim <= 128 ? 4 : 8;
     const int ct = vdim <= 32 ? 2 : vdim <= 64 ? 4 : vdim <= 128 ? 8 : 16;
     if (ma_lds_bytes(ks, ct, false) <= 160 * 1024) {
-      const bool split = max_q <= 1 && R <= 16;           // one token per request: the wavefronts split the window
+      // one token per request: the wavefronts split the window (where four staging areas fit the LDS)
+      const bool split = max_q <= 1 && R <= 16 && ma_lds_bytes(ks, ct, true) <= 156 * 1024;
       const int TQm = max_q <= 1 ? 1 : 64 / R;
+      // ... and with few requests several workgroups do, when the caller brought room for their shares
+      int ksplit = split ? window_attn_key_splits(tokens, kv_heads) : 1;
+      if (ksplit > 1 && (!workspace || workspace_bytes < (size_t)tokens * heads * ksplit * (vdim + 2) * sizeof(float)))
+        ksplit = 1;
       WAttnArgs pm{q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride, tokens, heads,
                    kv_heads, dim, vdim, block_size, window, TQm, MA_KEYS, softcap, out_scale, cw, v_col, distance_term, sink,
-                   gate, gate_row_stride};
-      dim3 gridm((unsigned)((tokens + TQm - 1) / TQm), (unsigned)kv_heads);
+                   gate, gate_row_stride, ksplit, reinterpret_cast<float*>(workspace)};
+      dim3 gridm((unsigned)((tokens + TQm - 1) / TQm), (unsigned)kv_heads, (unsigned)ksplit);
       hipStream_t st = (hipStream_t)stream;
       const hipError_t e = ks == 2 ? launch_window_mfma<2>(pm, ct, split, gridm, st)
                            : ks == 4 ? launch_window_mfma<4>(pm, ct, split, gridm, st)
@@ -591,6 +653,10 @@ extern "C" int nv_paged_softmax_attn(const float* q, const void* cache, const in
       if (e != hipSuccess) {
         nv_set_error("nv_window_attn: %s", hipGetErrorString(e));
         return NV_ERR_LAUNCH;
+      }
+      if (ksplit > 1) {
+        window_attn_join_kernel<<<dim3((unsigned)((tokens * heads + 3) / 4)), dim3(256), 0, st>>>(pm);
+        NV_CHECK_LAUNCH();
       }
       return NV_OK;
     }
@@ -608,7 +674,7 @@ extern "C" int nv_paged_softmax_attn(const float* q, const void* cache, const in
   const int64_t tiles = (tokens + TQ - 1) / TQ;
   WAttnArgs p{q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride, tokens, heads,
               kv_heads, dim, vdim, block_size, window, TQ, TK, softcap, out_scale, cw, v_col, distance_term, sink, gate,
-              gate_row_stride};
+              gate_row_stride, 1, nullptr};
   dim3 grid((unsigned)tiles, (unsigned)kv_heads);
   NV_DISPATCH_T(dtype, window_attn_kernel<T><<<grid, dim3(256), need(TQ, TK), (hipStream_t)stream>>>(p));
   NV_CHECK_LAUNCH();

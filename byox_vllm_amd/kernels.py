@@ -852,11 +852,16 @@ def paged_softmax_attn(q, cache, block_tables, cu_q, past_lens, seq_of_token, ma
     assert sink is None or (sink.dtype == cache.dtype and sink.numel() == heads and sink.is_contiguous())
     assert gate is None or (gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.size(0) == T
                             and gate.size(1) >= heads * vdim)
+    # steps of one token per request: room for the shares of several workgroups per token (sized before graph capture
+    # by the warm-up run of the same shape)
+    nbytes = lib().nv_paged_softmax_attn_workspace_bytes(T, max_q, heads, kv_heads, vdim) if cache.dtype == torch.bfloat16 else 0
+    ws = workspace(nbytes, q.device, "paged_softmax_attn") if nbytes else None
     check(lib().nv_paged_softmax_attn(ptr(q), ptr(cache), ptr(block_tables), block_tables.size(1), ptr(cu_q),
                                       ptr(past_lens), ptr(seq_of_token), ptr(out), out.stride(0), T, max_q, heads, kv_heads,
                                       dim, vdim, block_size, window, float(softcap or 0.0), out_scale, int(distance_term),
                                       int(values_are_keys), ptr(sink), ptr(gate),
-                                      gate.stride(0) if gate is not None else 0, _code32(cache.dtype), stream()),
+                                      gate.stride(0) if gate is not None else 0, ptr(ws), nbytes, _code32(cache.dtype),
+                                      stream()),
           "nv_paged_softmax_attn")
     return out
 

@@ -475,8 +475,12 @@ int nv_paged_softmax_attn(const float* q, const void* cache, const int32_t* bloc
                           const int32_t* cu_q, const int32_t* past_lens, const int32_t* seq_of_token, void* out,
                           int64_t out_row_stride, int64_t tokens, int max_q, int heads, int kv_heads, int dim, int vdim,
                           int block_size, int window, float softcap, float out_scale, int distance_term,
-                          int values_are_keys, const void* sink, const float* gate, int64_t gate_row_stride, int dtype,
-                          nv_stream_t stream);
+                          int values_are_keys, const void* sink, const float* gate, int64_t gate_row_stride,
+                          void* workspace, size_t workspace_bytes, int dtype, nv_stream_t stream);
+/* Bytes of scratch with which a launch of one token per request (max_q 1) lets several workgroups share a token's
+ * keys (their shares are joined by a second kernel); 0 where that does not apply.  Without the scratch (null) the
+ * launch keeps one workgroup per token and key/value head. */
+size_t nv_paged_softmax_attn_workspace_bytes(int64_t tokens, int max_q, int heads, int kv_heads, int vdim);
 
 /* ---- recurrences with an fp32 state per request (csrc/scan.hip) ----
  * nv_causal_conv: per-channel causal convolution over fp32 rows; state [slots, taps - 1, channels] keeps the last
