@@ -505,12 +505,20 @@ __global__ __launch_bounds__(256) void window_attn_join_kernel(WAttnArgs p) {
   const int lane = threadIdx.x & 63, dv = p.dv, h = (int)(row % p.H);
   const int64_t t = row / p.H;
   const float* src = p.partial + row * p.ksplit * (dv + 2);
-  float m = -INFINITY;
-  for (int z = 0; z < p.ksplit; ++z) m = fmaxf(m, src[z * (dv + 2) + dv]);
-  float l = 0.0f;
-  for (int z = 0; z < p.ksplit; ++z) {
-    const float mz = src[z * (dv + 2) + dv];
-    l += mz == -INFINITY ? 0.0f : src[z * (dv + 2) + dv + 1] * __expf(mz - m);
+  // all maxima and sums first (at most 8 shares: the loads go out together), then one weight per share
+  float mz[8], wz[8];
+  float m = -INFINITY, l = 0.0f;
+#pragma unroll
+  for (int z = 0; z < 8; ++z) {
+    mz[z] = z < p.ksplit ? src[z * (dv + 2) + dv] : -INFINITY;
+    wz[z] = z < p.ksplit ? src[z * (dv + 2) + dv + 1] : 0.0f;
+    m = fmaxf(m, mz[z]);
+  }
+#pragma unroll
+  for (int z = 0; z < 8; ++z) {
+    const float f = mz[z] == -INFINITY ? 0.0f : __expf(mz[z] - m);
+    l += wz[z] * f;
+    wz[z] = f;
   }
   const bf16_t* sink = reinterpret_cast<const bf16_t*>(p.sink);
   float f, den;
@@ -518,10 +526,9 @@ __global__ __launch_bounds__(256) void window_attn_join_kernel(WAttnArgs p) {
   bf16_t* out = reinterpret_cast<bf16_t*>(p.out) + t * p.out_rs + h * dv;
   for (int e = lane; e < dv; e += 64) {
     float o = 0.0f;
-    for (int z = 0; z < p.ksplit; ++z) {
-      const float mz = src[z * (dv + 2) + dv];
-      o += mz == -INFINITY ? 0.0f : src[z * (dv + 2) + e] * __expf(mz - m);
-    }
+#pragma unroll
+    for (int z = 0; z < 8; ++z)
+      if (z < p.ksplit) o += src[z * (dv + 2) + e] * wz[z];
     float v = o * f * p.out_scale / den;
     if (p.gate) v *= sigmoid_f32(p.gate[t * p.gate_rs + h * dv + e]);
     out[e] = (bf16_t)v;
