@@ -9,8 +9,8 @@ feeds both sublayers.  The mixer of a layer is one of
 The feed-forward is a mixture of experts (clamped gated units, softmax over all experts renormalised over the chosen
 ones, layers/moe.py) or absent.  Norms are RMS norms with weights stored around zero (layers/hyper.py with one stream).
 A span of layers ``loop.start .. loop.stop - 1`` runs ``loop.times`` times in a row with the same weights; before the
-first layer of every pass the residual is replaced by W_in [x; x0], x0 being the embedding's output, and every pass has
-its own cache rows and state.  The head is the embedding table.
+first layer of every repetition the residual is replaced by W_in [x; x0], x0 being the embedding's output, and the
+repetitions keep separate cache rows and states.  The head is the embedding table.
 
 config.json: {"architecture": "Zamusun", "vocab", "width", "norm": {"eps"}, "loop": {"start", "stop", "times"} | absent,
 "layers": [{"type", "mixer": {...}, "mlp": {"kind": "moe", "router": {"experts", "top"}, "expert": {"ff", "limit"}} |
