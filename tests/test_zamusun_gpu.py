@@ -476,10 +476,35 @@ def setup(request):
     torch.manual_seed(99)
     reqs = {"a": torch.randint(0, cfg["vocab"], (83,)).tolist(), "b": torch.randint(0, cfg["vocab"], (31,)).tolist(),
             "c": torch.randint(0, cfg["vocab"], (2,)).tolist(), "d": torch.randint(0, cfg["vocab"], (50,)).tolist()}
-    want = {n: O.forward(t, weights, cfg).float() for n, t in reqs.items()}
+    want, clear = {}, {}
+    for n, t in reqs.items():
+        logits, gaps = _forward_with_router_gaps(t, weights, cfg)
+        want[n] = logits.float()
+        # tokens up to the first whose routers (any layer run) had a close call: no 16-bit rounding can change their experts
+        close = (gaps < 0.05).nonzero()
+        clear[n] = int(close[0]) if len(close) else len(t)
     engine = Engine(cfg, weights, dtype, blocks=12, slots=3)
+    engine.clear = clear
     whole = engine.replay(reqs, [[(n, len(t))] for n, t in reqs.items()])
     return cfg, weights, dtype, reqs, want, engine, whole
+
+
+def _forward_with_router_gaps(tokens, weights, cfg):
+    """The oracle's logits and, per token, the smallest gap over all routers between the last chosen logit and the
+    first one left out."""
+    gaps, route = [], O.route
+
+    def recording(z, top):
+        ordered = z.sort(-1, descending=True).values
+        gaps.append(ordered[:, top - 1] - ordered[:, top] if top < z.shape[1] else torch.full((z.shape[0],), math.inf,
+                                                                                              dtype=F64))
+        return route(z, top)
+    O.route = recording
+    try:
+        logits = O.forward(tokens, weights, cfg)
+    finally:
+        O.route = route
+    return logits, (torch.stack(gaps).min(0).values if gaps else torch.full((len(tokens),), math.inf, dtype=F64))
 
 
 def _check(setup, got):
@@ -489,10 +514,13 @@ def _check(setup, got):
             assert row_error(got[n], want[n]) < F32_TOL, (n, row_error(got[n], want[n]))
             assert row_error(got[n], whole[n]) < SAME_TOL, n
         else:
-            # a router logit of random weights can lie inside the rounding of its 16-bit input: a twentieth of the rows
-            # may take another expert
+            # A router logit of random weights can lie inside the rounding of its 16-bit input; a token that takes
+            # another expert is off by much more than rounding, and so, less, are the tokens after it (states and keys
+            # carry it on).  Sharp where no router had a close call yet; after that a tenth of the rows may differ.
             err = row_errors(got[n], want[n])
-            assert float((err > BF16_TOL).float().mean()) <= 0.05 and float(err.median()) < BF16_TOL / 2, (n, err.max())
+            head = err[:engine.clear[n]]
+            assert head.numel() == 0 or float(head.max()) < BF16_TOL, (n, engine.clear[n], head.max())
+            assert float((err > BF16_TOL).float().mean()) <= 0.1 and float(err.median()) < BF16_TOL / 2, (n, err.max())
 
 
 def test_whole_prompts_match_the_oracle(setup):
