@@ -70,6 +70,7 @@ _PROTOS = {
                        _i64, _f, _i, _p]),
     "nv_embed_scale": (_i, [_p, _p, _p, _i64, _i, _i64, _f, _i, _p]),
     "nv_dyt_norm": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
+    "nv_gated_postnorm_add": (_i, [_p, _p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i, _f, _f, _i, _p]),
     "nv_rmsnorm_f32": (_i, [_p, _i64, _p, _p, _i64, _i64, _i, _f, _i, _p]),
     "nv_act_mul_f32": (_i, [_p, _p, _i64, _i, _i, _f, _i, _p]),
     "nv_act_f32": (_i, [_p, _p, _i64, _i, _p, _f, _i, _p]),
@@ -79,8 +80,8 @@ _PROTOS = {
     "nv_matrix_memory": (_i, [_p, _i64, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _i, _f, _f,
                               _i, _p]),
     "nv_residual_pair": (_i, [_p, _p, _i64, _p, _p, _i64, _i, _i, _p]),
-    "nv_latent_kv_store": (_i, [_p, _i64, _p, _p, _p, _f, _p, _p, _i64, _i, _i, _i, _f, _i, _p]),
-    "nv_latent_q_rope": (_i, [_p, _i64, _p, _p, _f, _p, _i64, _i, _i, _i, _i, _i, _i, _p]),
+    "nv_latent_kv_store": (_i, [_p, _i64, _p, _p, _p, _f, _p, _p, _i64, _i, _i, _i, _i, _f, _i, _p]),
+    "nv_latent_q_rope": (_i, [_p, _i64, _p, _p, _f, _p, _i64, _i, _i, _i, _i, _i, _i, _i, _p]),
     "nv_latent_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _i, _f, _i, _p]),
     "nv_moe_route": (_i, [_p, _i64, _p, _p, _i64, _i, _i, _i, _p]),
     "nv_moe_sort": (_i, [_p, _i64, _i, _i, _p, _p, _p, _p]),
@@ -92,11 +93,14 @@ _PROTOS = {
     "nv_qk_norm_store": (_i, [_p, _p, _i64, _i, _i, _i, _p, _p, _p, _f, _f, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _p]),
     "nv_window_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _p]),
     "nv_qk_store": (_i, [_p, _p, _i64, _i, _i, _i, _p, _p, _p, _p, _f, _i, _f, _f, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _p]),
-    "nv_paged_softmax_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _i,
-                                   _p, _p, _i64, _p, _sz, _i, _p]),
+    "nv_paged_softmax_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i64, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i,
+                                   _i, _p, _p, _i64, _i, _p, _sz, _i, _p]),
+    "nv_qk_rotate_store": (_i, [_p, _p, _i64, _i, _i, _i, _p, _p, _i, _p, _p, _f, _i, _p, _i, _f, _p, _i64, _p, _f, _f, _p,
+                                _p, _p, _i64, _i, _i, _i, _i, _i, _p]),
     "nv_paged_softmax_attn_workspace_bytes": (_sz, [_i64, _i, _i, _i, _i]),
     "nv_causal_conv": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _i, _i, _i, _i, _p]),
     "nv_rglru_scan": (_i, [_p, _i64, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _i, _f, _f, _i, _p]),
+    "nv_mingru_scan": (_i, [_p, _i64, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _i, _p]),
     "nv_ssd_scan": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _sz, _i,
                          _p]),
     "nv_ssd_scan_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),

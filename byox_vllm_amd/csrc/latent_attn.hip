@@ -8,8 +8,9 @@
 //   nv_latent_q_rope   : rotation of the per-head query parts into the absorbed-query buffer
 //   nv_latent_attn     : sliding-window softmax attention, one workgroup per (token, group of heads)
 //
-// Rotation ("rotate half"): dimension i pairs with i + dims/2; the angle is position * inv_freq[i] in fp32, and both
-// cosine and sine are multiplied by `mscale` (the caller folds frequency scaling into inv_freq and mscale).
+// Rotation: dimension i pairs with i + dims/2 ("rotate half"), or with `interleaved` dimension 2i with 2i + 1; the angle
+// is position * inv_freq[i] in fp32, and both cosine and sine are multiplied by `mscale` (the caller folds frequency
+// scaling into inv_freq and mscale).
 #include "anyt.h"
 
 namespace {
@@ -21,7 +22,7 @@ __global__ __launch_bounds__(256) void latent_kv_store_kernel(const float* __res
                                                               const float* __restrict__ inv_freq, float mscale,
                                                               const int32_t* __restrict__ slot_mapping,
                                                               T* __restrict__ cache, int rank, int rot_dim, int rot_dims,
-                                                              float eps) {
+                                                              float eps, int interleaved) {
   __shared__ float red[32];
   const int64_t t = blockIdx.x;
   const int32_t slot = slot_mapping[t];
@@ -38,11 +39,12 @@ __global__ __launch_bounds__(256) void latent_kv_store_kernel(const float* __res
   for (int j = threadIdx.x; j < rot_dim; j += blockDim.x) {
     float v = row[rank + j];
     if (j < rot_dims) {
-      const int i = j < half ? j : j - half;
+      const bool first = interleaved ? (j & 1) == 0 : j < half;
+      const int i = interleaved ? j >> 1 : (first ? j : j - half);
       const float a = pos * inv_freq[i];
       const float cs = cosf(a) * mscale, sn = sinf(a) * mscale;
-      const float other = row[rank + (j < half ? j + half : j - half)];
-      v = j < half ? v * cs - other * sn : v * cs + other * sn;
+      const float other = row[rank + (interleaved ? j ^ 1 : (first ? j + half : j - half))];
+      v = first ? v * cs - other * sn : v * cs + other * sn;
     }
     st_f32<T>(dst + rank + j, v);
   }
@@ -54,7 +56,7 @@ __global__ __launch_bounds__(256) void latent_q_rope_kernel(const T* __restrict_
                                                             const int64_t* __restrict__ positions,
                                                             const float* __restrict__ inv_freq, float mscale,
                                                             float* __restrict__ qa, int H, int dim, int rot_dim,
-                                                            int rot_dims, int rank) {
+                                                            int rot_dims, int rank, int interleaved) {
   const int64_t t = blockIdx.x;
   const float pos = (float)positions[t];
   const int half = rot_dims / 2;
@@ -63,11 +65,12 @@ __global__ __launch_bounds__(256) void latent_q_rope_kernel(const T* __restrict_
     const T* src = q + t * q_rs + (int64_t)h * (dim + rot_dim) + dim;
     float v = ld_f32<T>(src + j);
     if (j < rot_dims) {
-      const int i = j < half ? j : j - half;
+      const bool first = interleaved ? (j & 1) == 0 : j < half;
+      const int i = interleaved ? j >> 1 : (first ? j : j - half);
       const float a = pos * inv_freq[i];
       const float cs = cosf(a) * mscale, sn = sinf(a) * mscale;
-      const float other = ld_f32<T>(src + (j < half ? j + half : j - half));
-      v = j < half ? v * cs - other * sn : v * cs + other * sn;
+      const float other = ld_f32<T>(src + (interleaved ? j ^ 1 : (first ? j + half : j - half)));
+      v = first ? v * cs - other * sn : v * cs + other * sn;
     }
     qa[(t * H + h) * (rank + rot_dim) + rank + j] = v;
   }
@@ -396,8 +399,8 @@ hipError_t launch_mfma_attn(const MfmaAttnArgs& q, dim3 grid, size_t lds, hipStr
 
 extern "C" int nv_latent_kv_store(const float* kv, int64_t kv_row_stride, const void* norm_w, const int64_t* positions,
                                   const float* inv_freq, float mscale, const int32_t* slot_mapping, void* cache,
-                                  int64_t tokens, int rank, int rot_dim, int rot_dims, float eps, int dtype,
-                                  nv_stream_t stream) {
+                                  int64_t tokens, int rank, int rot_dim, int rot_dims, int interleaved, float eps,
+                                  int dtype, nv_stream_t stream) {
   NV_CHECK_ARG(kv && norm_w && positions && inv_freq && slot_mapping && cache, "nv_latent_kv_store: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_latent_kv_store: bad dtype %d", dtype);
   NV_CHECK_ARG(tokens >= 0 && rank > 0 && rot_dim >= 0 && rot_dims >= 0 && rot_dims <= rot_dim && rot_dims % 2 == 0,
@@ -405,21 +408,22 @@ extern "C" int nv_latent_kv_store(const float* kv, int64_t kv_row_stride, const 
   if (tokens == 0) return NV_OK;
   NV_DISPATCH_T(dtype, latent_kv_store_kernel<T><<<dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream>>>(
                            kv, kv_row_stride, (const T*)norm_w, positions, inv_freq, mscale, slot_mapping, (T*)cache,
-                           rank, rot_dim, rot_dims, eps));
+                           rank, rot_dim, rot_dims, eps, interleaved));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }
 
 extern "C" int nv_latent_q_rope(const void* q, int64_t q_row_stride, const int64_t* positions, const float* inv_freq,
                                 float mscale, float* qa, int64_t tokens, int heads, int dim, int rot_dim, int rot_dims,
-                                int rank, int dtype, nv_stream_t stream) {
+                                int interleaved, int rank, int dtype, nv_stream_t stream) {
   NV_CHECK_ARG(q && positions && inv_freq && qa, "nv_latent_q_rope: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_latent_q_rope: bad dtype %d", dtype);
   NV_CHECK_ARG(tokens >= 0 && heads > 0 && dim >= 0 && rot_dim >= 0 && rot_dims <= rot_dim && rot_dims % 2 == 0 && rank > 0,
                "nv_latent_q_rope: bad shape");
   if (tokens == 0 || rot_dim == 0) return NV_OK;
   NV_DISPATCH_T(dtype, latent_q_rope_kernel<T><<<dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream>>>(
-                           (const T*)q, q_row_stride, positions, inv_freq, mscale, qa, heads, dim, rot_dim, rot_dims, rank));
+                           (const T*)q, q_row_stride, positions, inv_freq, mscale, qa, heads, dim, rot_dim, rot_dims, rank,
+                           interleaved));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void linear_kernel(LinArgs p) {
       } else if constexpr (EPI == EPI_SOFTCAP) {
         v = p.epi_c * tanhf(v / p.epi_c);
       } else if constexpr (EPI == EPI_ROW_GATE) {
-        v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + z]);
+        v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + (p.act ? (int64_t)z * p.N + n : z)]);
       } else if constexpr (EPI == EPI_ACT) {
         v = unary_act(v, p.act, p.epi_ptr, p.epi_c);
       }
@@ -305,7 +305,7 @@ __global__ __launch_bounds__(256) void linear_tile_kernel(LinArgs p) {
         } else if constexpr (EPI == EPI_SOFTCAP) {
           v = p.epi_c * tanhf(v / p.epi_c);
         } else if constexpr (EPI == EPI_ROW_GATE) {
-          v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + z]);
+          v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + (p.act ? (int64_t)z * p.N + n : z)]);
         } else if constexpr (EPI == EPI_ACT) {
           v = unary_act(v, p.act, p.epi_ptr, p.epi_c);
         }
@@ -417,7 +417,7 @@ __global__ __launch_bounds__(256) void linear_fewrow_kernel(LinArgs p) {
       } else if constexpr (EPI == EPI_SOFTCAP) {
         v = p.epi_c * tanhf(v / p.epi_c);
       } else if constexpr (EPI == EPI_ROW_GATE) {
-        v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + z]);
+        v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + (p.act ? (int64_t)z * p.N + n : z)]);
       } else if constexpr (EPI == EPI_ACT) {
         v = unary_act(v, p.act, p.epi_ptr, p.epi_c);
       }

@@ -51,6 +51,44 @@ __global__ __launch_bounds__(256) void rmsnorm_f32_kernel(const float* __restric
   for (int j = threadIdx.x; j < n; j += blockDim.x) st_f32<T>(out + r * out_rs + j, xr[j] * inv * ld_f32<T>(w + j));
 }
 
+// Post-norm residual with a gate: x[t] += mult * (g / sqrt(mean(g^2) + eps)) * w, g = y[t] * sigmoid(gate[t] + gate_bias)
+// (no gate: g = y); the new row is also written in the storage type for the products that read the residual.  Without y
+// the row is only copied.
+template <typename T>
+__global__ __launch_bounds__(256) void gated_postnorm_add_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                                 int64_t y_rs, const float* __restrict__ gate,
+                                                                 int64_t gate_rs, const T* __restrict__ gate_bias,
+                                                                 const T* __restrict__ w, T* __restrict__ out_t,
+                                                                 int64_t out_rs, int n, float eps, float mult) {
+  __shared__ float red[32];
+  const int64_t t = blockIdx.x;
+  float* xr = x + t * n;
+  if (y == nullptr) {
+    if (out_t)
+      for (int j = threadIdx.x; j < n; j += blockDim.x) st_f32<T>(out_t + t * out_rs + j, xr[j]);
+    return;
+  }
+  const float* yr = y + t * y_rs;
+  const float* gr = gate ? gate + t * gate_rs : nullptr;
+  auto gated = [&](int j) {
+    float v = yr[j];
+    if (gr) v *= sigmoid_f32(gr[j] + (gate_bias ? ld_f32<T>(gate_bias + j) : 0.0f));
+    return v;
+  };
+  float ss = 0.0f;
+  for (int j = threadIdx.x; j < n; j += blockDim.x) {
+    const float v = gated(j);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = mult / sqrtf(ss / (float)n + eps);
+  for (int j = threadIdx.x; j < n; j += blockDim.x) {
+    const float v = xr[j] + gated(j) * inv * ld_f32<T>(w + j);
+    xr[j] = v;
+    if (out_t) st_f32<T>(out_t + t * out_rs + j, v);
+  }
+}
+
 // out[t] = [x[t] | x0[t]] in the storage type; x takes delta first
 template <typename T>
 __global__ __launch_bounds__(256) void residual_pair_kernel(float* __restrict__ x, const float* __restrict__ delta,
@@ -235,6 +273,22 @@ extern "C" int nv_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* 
   if (rows == 0) return NV_OK;
   NV_DISPATCH_T(dtype, rmsnorm_f32_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
                            x, x_row_stride, (const T*)w, (T*)out, out_row_stride, n, eps));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_gated_postnorm_add(float* x, const float* y, int64_t y_row_stride, const float* gate,
+                                     int64_t gate_row_stride, const void* gate_bias, const void* w, void* out,
+                                     int64_t out_row_stride, int64_t rows, int n, float eps, float mult, int dtype,
+                                     nv_stream_t stream) {
+  NV_CHECK_ARG(x && (y == nullptr || w), "nv_gated_postnorm_add: null pointer");
+  NV_CHECK_ARG(y || out, "nv_gated_postnorm_add: nothing to do");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_gated_postnorm_add: bad dtype %d", dtype);
+  NV_CHECK_ARG(rows >= 0 && n > 0, "nv_gated_postnorm_add: bad shape");
+  if (rows == 0) return NV_OK;
+  NV_DISPATCH_T(dtype, gated_postnorm_add_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
+                           x, y, y_row_stride, gate, gate_row_stride, (const T*)gate_bias, (const T*)w, (T*)out,
+                           out_row_stride, n, eps, mult));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

@@ -3,9 +3,11 @@
 // tokens behind it) and leaving the state there, so a prompt, its portions and single decoded tokens go one way.
 //
 // causal_conv:  out[t][c] = act(bias[c] + sum_j w[c][j] * x[t - (taps - 1 - j)][c]); the slot keeps the last
-//               taps - 1 inputs of every channel.
+//               taps - 1 inputs of every channel.  act 2 adds the token's own input: out = x[t] + conv(x)[t].
 // rglru_scan:   a = exp(-c * sigmoid(gr) * softplus(lam)),  S = a S + sqrt(1 - a^2) * sigmoid(gi) * u,
 //               out = S * gelu_tanh(y) * out_scale: the real-gated linear recurrent unit of the Griffin block.
+// mingru_scan:  z = sigmoid(zl),  S = (1 - z) S + z c(u),  c(u) = u + 1/2 for u >= 0 and sigmoid(u) below,
+//               out = S * silu(g): the minimal gated recurrent unit, whose gates read the current token only.
 // ssd_scan:     per head, S [N, P]:  S = exp(-exp(A_log) dt) S + dt B x^T,  y = S^T C + D x,  dt = softplus(raw + bias);
 //               out = y * silu(z): the selective state-space recurrence of Mamba-2 in its token-by-token form.
 #include "anyt.h"
@@ -31,7 +33,7 @@ struct ConvArgs {
   int64_t of_rs;
   void* out_t;            // [tokens, ot_rs] in the storage type, or null
   int64_t ot_rs;
-  int C, taps, act;       // act 0: none, 1: SiLU
+  int C, taps, act;       // act 0: none, 1: SiLU, 2: none, and the token's own input is added to the result
 };
 
 // One thread per (token, channel).  Only a portion's first taps - 1 tokens need the slot; they are all served by the
@@ -54,6 +56,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs p) {
   for (int j = 0; j < CONV_MAX_TAPS; ++j) wt[j] = j < taps ? ld_f32<T>(w + j) : 0.0f;
   auto emit = [&](int64_t tt, float v) {
     if (p.act == 1) v = silu_f32(v);
+    if (p.act == 2) v += p.x[tt * p.x_rs + c] + xb;
     if (p.out_f32) p.out_f32[tt * p.of_rs + c] = v;
     if (p.out_t) st_f32<T>(reinterpret_cast<T*>(p.out_t) + tt * p.ot_rs + c, v);
   };
@@ -116,27 +119,19 @@ struct RglruArgs {
 // A step of one token per request costs one run's walk; a prompt's walk is RG_CHUNKS times shorter than the prompt.
 constexpr int RG_CHUNKS = 16, RG_CH = 64;
 
-template <typename T>
-__global__ __launch_bounds__(RG_CHUNKS * RG_CH) void rglru_scan_kernel(RglruArgs p) {
+// the walk both gated recurrences share: step(t, a, b) gives the token's map S -> a S + b, emit(t, S) writes its output
+template <typename Step, typename Emit>
+__device__ __forceinline__ void affine_scan(const int32_t* cu_q, const int32_t* past, const int32_t* slots, float* state,
+                                            int C, Step step, Emit emit) {
   __shared__ float sA[RG_CHUNKS][RG_CH], sB[RG_CHUNKS][RG_CH];
   const int cx = threadIdx.x, j = threadIdx.y;
   const int ch = blockIdx.x * RG_CH + cx;
   const int b = blockIdx.y;
-  const int t0 = p.cu_q[b], t1 = p.cu_q[b + 1];
+  const int t0 = cu_q[b], t1 = cu_q[b + 1];
   if (t1 <= t0) return;
-  const bool on = ch < p.C;
+  const bool on = ch < C;
   const int len = (t1 - t0 + RG_CHUNKS - 1) / RG_CHUNKS;
   const int64_t c0 = min((int64_t)t1, (int64_t)t0 + (int64_t)j * len), c1 = min((int64_t)t1, c0 + len);
-  const float sp = on ? p.c * softplus_f32(ld_f32<T>(reinterpret_cast<const T*>(p.lam) + ch)) : 0.0f;
-  const int gcol = on ? (ch / p.bw) * 2 * p.bw + ch % p.bw : 0;
-  const float yb = (on && p.y_bias) ? ld_f32<T>(reinterpret_cast<const T*>(p.y_bias) + ch) : 0.0f;
-  auto step = [&](int64_t t, float& a, float& inp) {
-    const float gr = p.gates[t * p.g_rs + gcol], gi = p.gates[t * p.g_rs + gcol + p.bw];
-    const float log_a = -sp * sigmoid_f32(gr);
-    a = expf(log_a);
-    // sqrt(1 - a^2) through expm1: 1 - exp(2 log a) loses its digits when the decay is close to one
-    inp = sqrtf(-expm1f(2.0f * log_a)) * sigmoid_f32(gi) * p.u[t * p.u_rs + ch];
-  };
   float A = 1.0f, B = 0.0f;
   if (on && t1 - t0 > 1) {
     for (int64_t t = c0; t < c1; ++t) {
@@ -150,18 +145,72 @@ __global__ __launch_bounds__(RG_CHUNKS * RG_CH) void rglru_scan_kernel(RglruArgs
   sB[j][cx] = B;
   __syncthreads();
   if (!on) return;
-  float* slot = p.state + (int64_t)p.slots[b] * p.C + ch;
-  float S = p.past[b] == 0 ? 0.0f : *slot;
+  float* slot = state + (int64_t)slots[b] * C + ch;
+  float S = past[b] == 0 ? 0.0f : *slot;
   if (t1 - t0 > 1)
     for (int jj = 0; jj < j; ++jj) S = sA[jj][cx] * S + sB[jj][cx];
-  T* out = reinterpret_cast<T*>(p.out);
   for (int64_t t = c0; t < c1; ++t) {
     float a, inp;
     step(t, a, inp);
     S = a * S + inp;
-    st_f32<T>(out + t * p.out_rs + ch, S * gelu_tanh_f32(p.y[t * p.y_rs + ch] + yb) * p.out_scale);
+    emit(t, S);
   }
   if (c1 == t1 && c1 > c0) *slot = S;      // the run that holds the step's last token
+}
+
+template <typename T>
+__global__ __launch_bounds__(RG_CHUNKS * RG_CH) void rglru_scan_kernel(RglruArgs p) {
+  const int ch = blockIdx.x * RG_CH + threadIdx.x;
+  const bool on = ch < p.C;
+  const float sp = on ? p.c * softplus_f32(ld_f32<T>(reinterpret_cast<const T*>(p.lam) + ch)) : 0.0f;
+  const int gcol = on ? (ch / p.bw) * 2 * p.bw + ch % p.bw : 0;
+  const float yb = (on && p.y_bias) ? ld_f32<T>(reinterpret_cast<const T*>(p.y_bias) + ch) : 0.0f;
+  T* out = reinterpret_cast<T*>(p.out);
+  affine_scan(
+      p.cu_q, p.past, p.slots, p.state, p.C,
+      [&](int64_t t, float& a, float& inp) {
+        const float gr = p.gates[t * p.g_rs + gcol], gi = p.gates[t * p.g_rs + gcol + p.bw];
+        const float log_a = -sp * sigmoid_f32(gr);
+        a = expf(log_a);
+        // sqrt(1 - a^2) through expm1: 1 - exp(2 log a) loses its digits when the decay is close to one
+        inp = sqrtf(-expm1f(2.0f * log_a)) * sigmoid_f32(gi) * p.u[t * p.u_rs + ch];
+      },
+      [&](int64_t t, float S) {
+        st_f32<T>(out + t * p.out_rs + ch, S * gelu_tanh_f32(p.y[t * p.y_rs + ch] + yb) * p.out_scale);
+      });
+}
+
+struct MinGruArgs {
+  const float* proj;      // [tokens, proj_rs] fp32 projections: update-gate logits, candidates and output-gate logits
+  int64_t proj_rs;
+  int z_off, u_off, g_off;   // at these columns, C of each
+  const void* z_bias;     // [C] or null
+  const void* u_bias;     // [C] or null
+  float* state;           // [slots, C]
+  const int32_t* cu_q;
+  const int32_t* past;
+  const int32_t* slots;
+  void* out;              // [tokens, out_rs]
+  int64_t out_rs;
+  int C;
+};
+
+template <typename T>
+__global__ __launch_bounds__(RG_CHUNKS * RG_CH) void mingru_scan_kernel(MinGruArgs p) {
+  const int ch = blockIdx.x * RG_CH + threadIdx.x;
+  const bool on = ch < p.C;
+  const float zb = (on && p.z_bias) ? ld_f32<T>(reinterpret_cast<const T*>(p.z_bias) + ch) : 0.0f;
+  const float ub = (on && p.u_bias) ? ld_f32<T>(reinterpret_cast<const T*>(p.u_bias) + ch) : 0.0f;
+  T* out = reinterpret_cast<T*>(p.out);
+  affine_scan(
+      p.cu_q, p.past, p.slots, p.state, p.C,
+      [&](int64_t t, float& a, float& inp) {
+        const float* row = p.proj + t * p.proj_rs;
+        const float zl = row[p.z_off + ch] + zb, u = row[p.u_off + ch] + ub;
+        a = sigmoid_f32(-zl);                      // 1 - sigmoid(zl), without the cancellation
+        inp = sigmoid_f32(zl) * (u >= 0.0f ? u + 0.5f : sigmoid_f32(u));
+      },
+      [&](int64_t t, float S) { st_f32<T>(out + t * p.out_rs + ch, S * silu_f32(p.proj[t * p.proj_rs + p.g_off + ch])); });
 }
 
 struct SsdArgs {
@@ -331,7 +380,7 @@ extern "C" int nv_causal_conv(const float* x, const void* x_bias, int64_t x_row_
                "nv_causal_conv: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_causal_conv: bad dtype %d", dtype);
   NV_CHECK_ARG(tokens >= 0 && tokens < (1ll << 31) && channels > 0 && taps >= 1 && taps <= CONV_MAX_TAPS &&
-                   (act == 0 || act == 1),
+                   act >= 0 && act <= 2,
                "nv_causal_conv: bad shape (taps up to %d)", CONV_MAX_TAPS);
   if (tokens == 0) return NV_OK;
   ConvArgs p{x, x_bias, x_row_stride, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, out_f32, out_f32_row_stride,
@@ -356,6 +405,23 @@ extern "C" int nv_rglru_scan(const float* u, int64_t u_row_stride, const float* 
               out_row_stride, channels, block_width, c, out_scale};
   NV_DISPATCH_T(dtype, rglru_scan_kernel<T><<<dim3((unsigned)((channels + RG_CH - 1) / RG_CH), (unsigned)num_seqs),
                                               dim3(RG_CH, RG_CHUNKS), 0, (hipStream_t)stream>>>(p));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_mingru_scan(const float* proj, int64_t proj_row_stride, int z_off, int u_off, int g_off,
+                              const void* z_bias, const void* u_bias, float* state, const int32_t* cu_q,
+                              const int32_t* past_lens, const int32_t* state_slots, void* out, int64_t out_row_stride,
+                              int num_seqs, int channels, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(proj && state && cu_q && past_lens && state_slots && out, "nv_mingru_scan: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_mingru_scan: bad dtype %d", dtype);
+  NV_CHECK_ARG(num_seqs >= 0 && num_seqs <= 65535 && channels > 0 && z_off >= 0 && u_off >= 0 && g_off >= 0,
+               "nv_mingru_scan: bad shape");
+  if (num_seqs == 0) return NV_OK;
+  MinGruArgs p{proj, proj_row_stride, z_off, u_off, g_off, z_bias, u_bias, state, cu_q, past_lens, state_slots, out,
+               out_row_stride, channels};
+  NV_DISPATCH_T(dtype, mingru_scan_kernel<T><<<dim3((unsigned)((channels + RG_CH - 1) / RG_CH), (unsigned)num_seqs),
+                                               dim3(RG_CH, RG_CHUNKS), 0, (hipStream_t)stream>>>(p));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

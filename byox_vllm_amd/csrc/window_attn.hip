@@ -5,12 +5,17 @@
 // scale and per-head temperature (qk_norm_store below), so the kernel's own arithmetic is the dot product, the cap,
 // the distance term and the softmax, all in fp32.  Options of a design: no distance term; a sink, one learned logit per
 // query head that joins the softmax's denominator without a key or a value; values that ARE the keys (rows [k: G * d]
-// only, read twice); a sigmoid output gate from fp32 logits laid out like the output.
+// only, read twice); a sigmoid output gate from fp32 logits laid out like the output, or one logit per head; chunks, in
+// which a query sees the keys j <= i of its own chunk only (floor(i / chunk) == floor(j / chunk), counted from the
+// sequence's first position).
 //
 // qk_norm_store: per token, RMS norm over each query and key head (one weight vector shared by the heads), the query
 // scaled by scale * temp[h] and left in fp32, the normalised key and the value written to the token's cache row
 // [k: G * d | v: G * dv] in the storage type.  The norms may be absent (null weights: the projection as it is), and
 // the query may carry a temperature that grows with the position p: 1 + coef * ln(floor((p + 1) / every) + 1).
+// Further options: one root mean square over all heads of q (and of k) with a weight per number; a rotation of the first
+// rot_dims numbers of every head after the norm (dimension i with i + rot_dims / 2, angle position * inv_freq[i]); values
+// blended with another layer's values of the same token, v <- (1 - lam) v + lam v_first, before they are stored.
 //
 // window_attn_kernel: a workgroup owns TQ consecutive tokens of the packed batch and one key/value head, i.e. up to
 // TQ * (H / G) query rows that read the same keys; tokens of different requests inside the tile are served one request
@@ -24,10 +29,10 @@ struct QkArgs {
   const void* bias;       // [proj columns] added to the projections (same column offsets), or null
   int64_t proj_rs;
   int q_off, k_off, v_off;
-  const void* qn;         // [d] query norm weight
-  const void* kn;         // [d]
+  const void* qn;         // query norm weight: [d] shared by the heads, or [H * d] when norm_whole
+  const void* kn;         // [d] or [G * d]
   const void* temp;       // [H] or null
-  const int64_t* positions;   // [tokens], read when temp_every > 0
+  const int64_t* positions;   // [tokens], read when temp_every > 0 or rot_dims > 0
   float temp_coef;
   int temp_every;         // 0: no position temperature
   const int32_t* slot_mapping;   // [tokens] cache row of each token, -1: none
@@ -35,10 +40,18 @@ struct QkArgs {
   float* q_out;           // [tokens, H * d]
   int H, G, d, dv;
   float scale, eps;
+  int norm_whole;         // 1: one root mean square over all H * d query numbers (and over all G * d key numbers)
+  const float* inv_freq;  // [rot_dims / 2] rotation frequencies, read when rot_dims > 0
+  int rot_dims;           // the first rot_dims numbers of every head are rotated, dimension i with i + rot_dims / 2
+  float mscale;           // multiplies cosine and sine
+  const float* v_first;   // [tokens, v_first_rs] values to blend in, or null
+  int64_t v_first_rs;
+  const void* vmix;       // one number lam: v <- (1 - lam) v + lam v_first
 };
 
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_store_kernel(QkArgs p) {
+  __shared__ float red[32];
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const float* row = p.proj + t * p.proj_rs;
@@ -51,12 +64,29 @@ __global__ __launch_bounds__(256) void qk_norm_store_kernel(QkArgs p) {
   const T* kn = reinterpret_cast<const T*>(p.kn);
   const T* temp = reinterpret_cast<const T*>(p.temp);
   const T* bias = reinterpret_cast<const T*>(p.bias);
+  const int half = p.rot_dims / 2;
+  const float pos = p.rot_dims > 0 ? (float)p.positions[t] : 0.0f;
+  float inv_q = 1.0f, inv_k = 1.0f;
+  if (qn && p.norm_whole) {
+    float sq = 0.0f, sk = 0.0f;
+    for (int e = threadIdx.x; e < p.H * p.d; e += blockDim.x) {
+      const float x = row[p.q_off + e] + (bias ? ld_f32<T>(bias + p.q_off + e) : 0.0f);
+      sq += x * x;
+    }
+    for (int e = threadIdx.x; e < p.G * p.d; e += blockDim.x) {
+      const float x = row[p.k_off + e] + (bias ? ld_f32<T>(bias + p.k_off + e) : 0.0f);
+      sk += x * x;
+    }
+    inv_q = 1.0f / sqrtf(block_sum(sq, red) / (float)(p.H * p.d) + p.eps);
+    inv_k = 1.0f / sqrtf(block_sum(sk, red) / (float)(p.G * p.d) + p.eps);
+  }
   for (int v = wv; v < p.H + p.G; v += nw) {
     const bool is_q = v < p.H;
-    const int col = is_q ? p.q_off + v * p.d : p.k_off + (v - p.H) * p.d;
+    const int hv = is_q ? v : v - p.H;
+    const int col = is_q ? p.q_off + hv * p.d : p.k_off + hv * p.d;
     const float* src = row + col;
-    float inv = 1.0f;
-    if (qn) {
+    float inv = is_q ? inv_q : inv_k;
+    if (qn && !p.norm_whole) {
       float ss = 0.0f;
       for (int e = lane; e < p.d; e += 64) {
         const float x = src[e] + (bias ? ld_f32<T>(bias + col + e) : 0.0f);
@@ -65,22 +95,38 @@ __global__ __launch_bounds__(256) void qk_norm_store_kernel(QkArgs p) {
       ss = wave_sum(ss);
       inv = 1.0f / sqrtf(ss / (float)p.d + p.eps);
     }
+    const T* nw_ = is_q ? qn : kn;
+    if (nw_ && p.norm_whole) nw_ += hv * p.d;
+    auto normed = [&](int e) {
+      const float x = src[e] + (bias ? ld_f32<T>(bias + col + e) : 0.0f);
+      return x * inv * (nw_ ? ld_f32<T>(nw_ + e) : 1.0f);
+    };
+    auto value = [&](int e) {      // normalised, then rotated
+      float x = normed(e);
+      if (e < p.rot_dims) {
+        const bool first = e < half;
+        const float a = pos * p.inv_freq[first ? e : e - half];
+        const float cs = cosf(a) * p.mscale, sn = sinf(a) * p.mscale;
+        const float other = normed(first ? e + half : e - half);
+        x = first ? x * cs - other * sn : x * cs + other * sn;
+      }
+      return x;
+    };
     if (is_q) {
       const float f = p.scale * (temp ? ld_f32<T>(temp + v) : 1.0f) * pos_temp;
-      for (int e = lane; e < p.d; e += 64) {
-        const float x = src[e] + (bias ? ld_f32<T>(bias + col + e) : 0.0f);
-        p.q_out[t * p.H * p.d + v * p.d + e] = x * inv * (qn ? ld_f32<T>(qn + e) : 1.0f) * f;
-      }
+      for (int e = lane; e < p.d; e += 64) p.q_out[t * p.H * p.d + v * p.d + e] = value(e) * f;
     } else if (crow) {
-      for (int e = lane; e < p.d; e += 64) {
-        const float x = src[e] + (bias ? ld_f32<T>(bias + col + e) : 0.0f);
-        st_f32<T>(crow + (v - p.H) * p.d + e, x * inv * (kn ? ld_f32<T>(kn + e) : 1.0f));
-      }
+      for (int e = lane; e < p.d; e += 64) st_f32<T>(crow + hv * p.d + e, value(e));
     }
   }
-  if (crow && p.dv > 0)
-    for (int e = threadIdx.x; e < p.G * p.dv; e += blockDim.x)
-      st_f32<T>(crow + p.G * p.d + e, row[p.v_off + e] + (bias ? ld_f32<T>(bias + p.v_off + e) : 0.0f));
+  if (crow && p.dv > 0) {
+    const float lam = p.v_first ? ld_f32<T>(reinterpret_cast<const T*>(p.vmix)) : 0.0f;
+    for (int e = threadIdx.x; e < p.G * p.dv; e += blockDim.x) {
+      float x = row[p.v_off + e] + (bias ? ld_f32<T>(bias + p.v_off + e) : 0.0f);
+      if (p.v_first) x = (1.0f - lam) * x + lam * p.v_first[t * p.v_first_rs + e];
+      st_f32<T>(crow + p.G * p.d + e, x);
+    }
+  }
 }
 
 struct WAttnArgs {
@@ -101,6 +147,8 @@ struct WAttnArgs {
   const void* sink;        // [H] logits that join the denominator, or null
   const float* gate;       // [tokens, gate_rs] logits whose sigmoid multiplies the output (head h at h * dv), or null
   int64_t gate_rs;
+  int gate_head;           // 1: one logit per head (head h at column h)
+  int chunk;               // > 0: a query sees only the keys of its own chunk, floor(i / chunk) == floor(j / chunk)
   int ksplit;              // SPLIT only: workgroups that share a token's keys (blockIdx.z); > 1: results go to `partial`
   float* partial;          // [tokens, H, ksplit, dv + 2]: unnormalised output, then maximum and sum
 };
@@ -155,7 +203,9 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WAttnArgs p) {
       sl[tid] = 0.0f;
     }
     __syncthreads();
-    const int lo = p.window > 0 ? max(0, p0 - p.window + 1) : 0, hi = p0 + nq - 1;
+    int lo = p.window > 0 ? max(0, p0 - p.window + 1) : 0;
+    if (p.chunk > 0) lo = max(lo, p0 / p.chunk * p.chunk);      // the tile's first token has the earliest chunk
+    const int hi = p0 + nq - 1;
     for (int j0 = lo; j0 <= hi; j0 += TK) {
       const int nk = min(TK, hi + 1 - j0);
       for (int i = tid; i < nk * (d + dv); i += 256) {
@@ -170,7 +220,7 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WAttnArgs p) {
         const int rr = i / TK, j = i % TK;
         const int pos = p0 + rr / R, kp = j0 + j;
         float s = -INFINITY;
-        if (j < nk && kp <= pos && (p.window <= 0 || pos - kp < p.window)) {
+        if (j < nk && kp <= pos && (p.window <= 0 || pos - kp < p.window) && (p.chunk <= 0 || kp >= pos / p.chunk * p.chunk)) {
           s = 0.0f;
           const float* qv = sq + rr * d;
           const float* kv = sk + j * dp;
@@ -218,7 +268,7 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WAttnArgs p) {
       float f, den;
       close_softmax(sm[rr], sl[rr], sink != nullptr, sink ? ld_f32<T>(sink + h) : 0.0f, f, den);
       float v = acc[i] * f / den * p.out_scale;
-      if (p.gate) v *= sigmoid_f32(p.gate[(ts + rr / R) * p.gate_rs + h * dv + e]);
+      if (p.gate) v *= sigmoid_f32(p.gate[(ts + rr / R) * p.gate_rs + (p.gate_head ? h : h * dv + e)]);
       st_f32<T>(out + (ts + rr / R) * p.out_rs + h * dv + e, v);
     }
     __syncthreads();
@@ -304,7 +354,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
       }
     }
     // the four accumulator rows of this lane
-    int pos[4];
+    int pos[4], kmin[4];      // kmin: first key of the row's chunk
     float slope[4], m_run[4], l_run[4];
     bool valid[4];
 #pragma unroll
@@ -312,6 +362,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
       const int rr = row0 + lg * 4 + r;
       valid[r] = rr < rows;
       pos[r] = p0 + rr / R;
+      kmin[r] = p.chunk > 0 ? pos[r] / p.chunk * p.chunk : 0;
       slope[r] = p.slope_on ? exp2f(-8.0f * (float)(g * R + rr % R + 1) / (float)p.H) : 0.0f;
       m_run[r] = -INFINITY;
       l_run[r] = 0.0f;
@@ -321,7 +372,9 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
     for (int ct = 0; ct < CT; ++ct) acc_o[ct] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     const int wpos_lo = p0 + row0 / R, wpos_hi = p0 + min(rows - 1, row0 + 15) / R;
 
-    const int lo = p.window > 0 ? max(0, p0 - p.window + 1) : 0, hi = p0 + nq - 1;
+    int lo = p.window > 0 ? max(0, p0 - p.window + 1) : 0;
+    if (p.chunk > 0) lo = max(lo, p0 / p.chunk * p.chunk);      // the tile's first token has the earliest chunk
+    const int hi = p0 + nq - 1;
     const int walkers = SPLIT ? 4 * p.ksplit : 1;          // wavefronts (of all workgroups) that share this token's keys
     for (int j0 = lo + (SPLIT ? ((int)blockIdx.z * 4 + wv) * MA_KEYS : 0); j0 <= hi; j0 += walkers * MA_KEYS) {
       if (stid < MA_KEYS) {
@@ -363,7 +416,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
       }
       sync();
       // keys this wavefront's rows can see: [wpos_lo - window + 1, wpos_hi]
-      const bool need = wave_on && j0 <= wpos_hi && (p.window <= 0 || j0 + MA_KEYS - 1 > wpos_lo - p.window);
+      const bool need = wave_on && j0 <= wpos_hi && (p.window <= 0 || j0 + MA_KEYS - 1 > wpos_lo - p.window) &&
+                        (p.chunk <= 0 || j0 + MA_KEYS - 1 >= wpos_lo / p.chunk * p.chunk);
       if (need) {
         f32x4 acc_s[4];
 #pragma unroll
@@ -386,7 +440,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
             float sc = acc_s[sub][r];
             if (p.softcap > 0.0f) sc = p.softcap * tanhf(sc / p.softcap);
             sc -= slope[r] * (float)dist;
-            const bool vis = valid[r] && dist >= 0 && (p.window <= 0 || dist < p.window);
+            const bool vis = valid[r] && dist >= 0 && (p.window <= 0 || dist < p.window) && kp >= kmin[r];
             sc = vis ? sc : -INFINITY;
             acc_s[sub][r] = sc;
             mt = fmaxf(mt, sc);
@@ -472,7 +526,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
         float f, den;
         close_softmax(m, l, sink != nullptr, sink ? ld_f32<bf16_t>(sink + h) : 0.0f, f, den);
         float v = o * f * p.out_scale / den;
-        if (p.gate) v *= sigmoid_f32(p.gate[(ts + rr / R) * p.gate_rs + h * dv + e]);
+        if (p.gate) v *= sigmoid_f32(p.gate[(ts + rr / R) * p.gate_rs + (p.gate_head ? h : h * dv + e)]);
         out[(ts + rr / R) * p.out_rs + h * dv + e] = (bf16_t)v;
       }
       __syncthreads();
@@ -486,11 +540,11 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
         close_softmax(m_run[r], l_run[r], sink != nullptr, sink ? ld_f32<bf16_t>(sink + h) : 0.0f, fs, den);
         const float f = p.out_scale * fs / den;
         bf16_t* orow = out + (ts + rr / R) * p.out_rs + h * dv;
-        const float* grow = p.gate ? p.gate + (ts + rr / R) * p.gate_rs + h * dv : nullptr;
+        const float* grow = p.gate ? p.gate + (ts + rr / R) * p.gate_rs + (p.gate_head ? h : h * dv) : nullptr;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
           const int e = ct * 16 + lc;
-          if (e < dv) orow[e] = (bf16_t)(acc_o[ct][r] * f * (grow ? sigmoid_f32(grow[e]) : 1.0f));
+          if (e < dv) orow[e] = (bf16_t)(acc_o[ct][r] * f * (grow ? sigmoid_f32(grow[p.gate_head ? 0 : e]) : 1.0f));
         }
       }
     }
@@ -530,7 +584,7 @@ __global__ __launch_bounds__(256) void window_attn_join_kernel(WAttnArgs p) {
     for (int z = 0; z < 8; ++z)
       if (z < p.ksplit) o += src[z * (dv + 2) + e] * wz[z];
     float v = o * f * p.out_scale / den;
-    if (p.gate) v *= sigmoid_f32(p.gate[t * p.gate_rs + h * dv + e]);
+    if (p.gate) v *= sigmoid_f32(p.gate[t * p.gate_rs + (p.gate_head ? h : h * dv + e)]);
     out[e] = (bf16_t)v;
   }
 }
@@ -589,15 +643,31 @@ extern "C" int nv_qk_store(const float* proj, const void* bias, int64_t proj_row
                            float temp_coef, int temp_every, float scale, float eps, const int32_t* slot_mapping,
                            void* cache, float* q_out, int64_t tokens, int heads, int kv_heads, int dim, int vdim, int dtype,
                            nv_stream_t stream) {
+  return nv_qk_rotate_store(proj, bias, proj_row_stride, q_off, k_off, v_off, q_norm, k_norm, 0, temp, positions, temp_coef,
+                            temp_every, nullptr, 0, 1.0f, nullptr, 0, nullptr, scale, eps, slot_mapping, cache, q_out,
+                            tokens, heads, kv_heads, dim, vdim, dtype, stream);
+}
+
+extern "C" int nv_qk_rotate_store(const float* proj, const void* bias, int64_t proj_row_stride, int q_off, int k_off,
+                                  int v_off, const void* q_norm, const void* k_norm, int norm_whole, const void* temp,
+                                  const int64_t* positions, float temp_coef, int temp_every, const float* inv_freq,
+                                  int rot_dims, float mscale, const float* v_first, int64_t v_first_row_stride,
+                                  const void* vmix, float scale, float eps, const int32_t* slot_mapping, void* cache,
+                                  float* q_out, int64_t tokens, int heads, int kv_heads, int dim, int vdim, int dtype,
+                                  nv_stream_t stream) {
   NV_CHECK_ARG(proj && slot_mapping && cache && q_out, "nv_qk_store: null pointer");
   NV_CHECK_ARG((q_norm == nullptr) == (k_norm == nullptr), "nv_qk_store: both norm weights or none");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_qk_store: bad dtype %d", dtype);
   NV_CHECK_ARG(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim >= 0,
                "nv_qk_store: bad shape");
   NV_CHECK_ARG(temp_every >= 0 && (temp_every == 0 || positions), "nv_qk_store: the position temperature needs positions");
+  NV_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dim && (rot_dims == 0 || (positions && inv_freq)),
+               "nv_qk_store: a rotation over %d of %d numbers needs positions and frequencies", rot_dims, dim);
+  NV_CHECK_ARG(!v_first || (vmix && vdim > 0), "nv_qk_store: blending values needs its weight");
   if (tokens == 0) return NV_OK;
   QkArgs p{proj, bias, proj_row_stride, q_off, k_off, v_off, q_norm, k_norm, temp, positions, temp_coef, temp_every,
-           slot_mapping, cache, q_out, heads, kv_heads, dim, vdim, scale, eps};
+           slot_mapping, cache, q_out, heads, kv_heads, dim, vdim, scale, eps, norm_whole, inv_freq, rot_dims, mscale,
+           v_first, v_first_row_stride, vmix};
   NV_DISPATCH_T(dtype, qk_norm_store_kernel<T><<<dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream>>>(p));
   NV_CHECK_LAUNCH();
   return NV_OK;
@@ -617,22 +687,23 @@ extern "C" int nv_window_attn(const float* q, const void* cache, const int32_t* 
                               int64_t out_row_stride, int64_t tokens, int max_q, int heads, int kv_heads, int dim, int vdim,
                               int block_size, int window, float softcap, float out_scale, int dtype, nv_stream_t stream) {
   return nv_paged_softmax_attn(q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride,
-                               tokens, max_q, heads, kv_heads, dim, vdim, block_size, window, softcap, out_scale, 1, 0,
-                               nullptr, nullptr, 0, nullptr, 0, dtype, stream);
+                               tokens, max_q, heads, kv_heads, dim, vdim, block_size, window, 0, softcap, out_scale, 1, 0,
+                               nullptr, nullptr, 0, 0, nullptr, 0, dtype, stream);
 }
 
 extern "C" int nv_paged_softmax_attn(const float* q, const void* cache, const int32_t* block_tables, int table_cols,
                                      const int32_t* cu_q, const int32_t* past_lens, const int32_t* seq_of_token, void* out,
                                      int64_t out_row_stride, int64_t tokens, int max_q, int heads, int kv_heads, int dim,
-                                     int vdim, int block_size, int window, float softcap, float out_scale, int distance_term,
-                                     int values_are_keys, const void* sink, const float* gate, int64_t gate_row_stride,
-                                     void* workspace, size_t workspace_bytes, int dtype, nv_stream_t stream) {
+                                     int vdim, int block_size, int window, int chunk, float softcap, float out_scale,
+                                     int distance_term, int values_are_keys, const void* sink, const float* gate,
+                                     int64_t gate_row_stride, int gate_per_head, void* workspace, size_t workspace_bytes,
+                                     int dtype, nv_stream_t stream) {
   NV_CHECK_ARG(q && cache && block_tables && cu_q && past_lens && seq_of_token && out, "nv_window_attn: null pointer");
   NV_CHECK_ARG(!values_are_keys || vdim == dim, "nv_window_attn: values that are the keys have the keys' size");
   const int cw = values_are_keys ? kv_heads * dim : kv_heads * (dim + vdim), v_col = values_are_keys ? 0 : kv_heads * dim;
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_window_attn: bad dtype %d", dtype);
   NV_CHECK_ARG(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 &&
-                   block_size > 0 && window >= 0 && table_cols > 0,
+                   block_size > 0 && window >= 0 && chunk >= 0 && table_cols > 0,
                "nv_window_attn: bad shape");
   if (tokens == 0) return NV_OK;
   const int R = heads / kv_heads;
@@ -651,7 +722,7 @@ extern "C" int nv_paged_softmax_attn(const float* q, const void* cache, const in
         ksplit = 1;
       WAttnArgs pm{q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride, tokens, heads,
                    kv_heads, dim, vdim, block_size, window, TQm, MA_KEYS, softcap, out_scale, cw, v_col, distance_term, sink,
-                   gate, gate_row_stride, ksplit, reinterpret_cast<float*>(workspace)};
+                   gate, gate_row_stride, gate_per_head, chunk, ksplit, reinterpret_cast<float*>(workspace)};
       dim3 gridm((unsigned)((tokens + TQm - 1) / TQm), (unsigned)kv_heads, (unsigned)ksplit);
       hipStream_t st = (hipStream_t)stream;
       const hipError_t e = ks == 2 ? launch_window_mfma<2>(pm, ct, split, gridm, st)
@@ -681,7 +752,7 @@ extern "C" int nv_paged_softmax_attn(const float* q, const void* cache, const in
   const int64_t tiles = (tokens + TQ - 1) / TQ;
   WAttnArgs p{q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride, tokens, heads,
               kv_heads, dim, vdim, block_size, window, TQ, TK, softcap, out_scale, cw, v_col, distance_term, sink, gate,
-              gate_row_stride, 1, nullptr};
+              gate_row_stride, gate_per_head, chunk, 1, nullptr};
   dim3 grid((unsigned)tiles, (unsigned)kv_heads);
   NV_DISPATCH_T(dtype, window_attn_kernel<T><<<grid, dim3(256), need(TQ, TK), (hipStream_t)stream>>>(p));
   NV_CHECK_LAUNCH();

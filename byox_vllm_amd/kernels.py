@@ -438,6 +438,7 @@ def stage_decode_packed(packed, bs, bt_cols, g, prev_tokens=None, block_size=0):
 
 EPI_NONE, EPI_GLU, EPI_SOFTCAP, EPI_ROW_GATE, EPI_ACT = 0, 1, 2, 3, 4
 ACT_SILU, ACT_GELU_TANH, ACT_XIELU, ACT_SCALE = 0, 1, 2, 3
+GATE_PER_NUMBER = 1  # EPI_ROW_GATE only (as ``act``): one gate logit per output number instead of one per row and batch
 GLU_CLAMPED = 2      # EPI_GLU only: g sigmoid(1.702 g) (u + 1) with g = min(gate, cap), u = clamp(up, -cap, cap)
 ROUTE_CHOSEN, ROUTE_ALL = 0, 1   # softmax over the chosen logits / over every expert, renormalised over the chosen
 
@@ -635,23 +636,26 @@ def residual_pair(x, x0, dtype, delta=None):
     return out
 
 
-def latent_kv_store(kv, norm_w, positions, inv_freq, mscale, slot_mapping, cache, rank, rot_dim, rot_dims, eps):
+def latent_kv_store(kv, norm_w, positions, inv_freq, mscale, slot_mapping, cache, rank, rot_dim, rot_dims, eps,
+                    interleaved=False):
+    """``interleaved``: dimension 2i turns with 2i + 1 instead of i with i + rot_dims / 2."""
     require_gpu(kv, "latent_kv_store")
     assert kv.dtype == torch.float32 and kv.stride(1) == 1 and kv.size(1) == rank + rot_dim
     assert positions.dtype == torch.int64 and slot_mapping.dtype == torch.int32 and inv_freq.dtype == torch.float32
     assert cache.is_contiguous() and cache.size(-1) == rank + rot_dim and cache.dtype == norm_w.dtype
     assert positions.numel() == slot_mapping.numel() == kv.size(0) and inv_freq.numel() * 2 >= rot_dims
     check(lib().nv_latent_kv_store(ptr(kv), kv.stride(0), ptr(norm_w), ptr(positions), ptr(inv_freq), mscale,
-                                   ptr(slot_mapping), ptr(cache), kv.size(0), rank, rot_dim, rot_dims, eps,
-                                   _code32(cache.dtype), stream()), "nv_latent_kv_store")
+                                   ptr(slot_mapping), ptr(cache), kv.size(0), rank, rot_dim, rot_dims, int(interleaved),
+                                   eps, _code32(cache.dtype), stream()), "nv_latent_kv_store")
 
 
-def latent_q_rope(q, positions, inv_freq, mscale, qa, heads, dim, rot_dim, rot_dims, rank):
+def latent_q_rope(q, positions, inv_freq, mscale, qa, heads, dim, rot_dim, rot_dims, rank, interleaved=False):
     require_gpu(q, "latent_q_rope")
     assert q.stride(1) == 1 and q.size(1) == heads * (dim + rot_dim) and qa.dtype == torch.float32 and qa.is_contiguous()
     assert qa.numel() == q.size(0) * heads * (rank + rot_dim) and positions.dtype == torch.int64
     check(lib().nv_latent_q_rope(ptr(q), q.stride(0), ptr(positions), ptr(inv_freq), mscale, ptr(qa), q.size(0), heads,
-                                 dim, rot_dim, rot_dims, rank, _code32(q.dtype), stream()), "nv_latent_q_rope")
+                                 dim, rot_dim, rot_dims, int(interleaved), rank, _code32(q.dtype), stream()),
+          "nv_latent_q_rope")
 
 
 def latent_attn(qa, cache, block_tables, cu_q, past_lens, seq_of_token, heads, rank, rot_dim, block_size, window, scale,
@@ -815,6 +819,43 @@ def window_attn(q, cache, block_tables, cu_q, past_lens, seq_of_token, max_q, he
     return out
 
 
+def qk_rotate_store(proj, offsets, positions, scale, slot_mapping, cache, heads, kv_heads, dim, vdim, *, q_norm=None,
+                    k_norm=None, eps=0.0, inv_freq=None, rot_dims=0, mscale=1.0, v_first=None, vmix=None, bias=None):
+    """fp32 projections [T, *] with q | k | v at ``offsets`` -> fp32 queries [T, heads * dim] times ``scale``; keys and
+    values go to cache rows [G * dim | G * vdim] of ``slot_mapping``.  ``q_norm`` [heads * dim] / ``k_norm``
+    [kv_heads * dim]: one RMS norm over all of a token's query numbers (and all of its key numbers) with a weight per
+    number.  ``rot_dims``: the first rot_dims numbers of every head turn by position * inv_freq[i], i with
+    i + rot_dims / 2.  ``v_first`` fp32 [T, G * vdim] (a column slice is fine): the stored values are
+    (1 - vmix) v + vmix v_first."""
+    require_gpu(proj, "qk_rotate_store")
+    T = proj.size(0)
+    assert proj.dtype == torch.float32 and proj.stride(1) == 1 and slot_mapping.dtype == torch.int32
+    assert slot_mapping.numel() == T and cache.is_contiguous() and cache.size(-1) == kv_heads * (dim + vdim)
+    assert positions.dtype == torch.int64 and positions.numel() == T and positions.is_contiguous()
+    q_off, k_off, v_off = offsets
+    need = max(q_off + heads * dim, k_off + kv_heads * dim, v_off + kv_heads * vdim)
+    assert need <= proj.size(1)
+    assert bias is None or (bias.dtype == cache.dtype and bias.is_contiguous() and need <= bias.numel() <= proj.size(1))
+    assert (q_norm is None) == (k_norm is None)
+    if q_norm is not None:
+        assert q_norm.numel() == heads * dim and k_norm.numel() == kv_heads * dim
+        assert q_norm.dtype == k_norm.dtype == cache.dtype and q_norm.is_contiguous() and k_norm.is_contiguous()
+    if rot_dims:
+        assert rot_dims % 2 == 0 and rot_dims <= dim and inv_freq.dtype == torch.float32 and inv_freq.is_contiguous()
+        assert inv_freq.numel() * 2 >= rot_dims and inv_freq.is_cuda
+    if v_first is not None:
+        assert v_first.dtype == torch.float32 and v_first.stride(1) == 1 and v_first.shape == (T, kv_heads * vdim)
+        assert vmix.dtype == cache.dtype and vmix.numel() == 1 and vmix.is_cuda
+    q = torch.empty(T, heads * dim, dtype=torch.float32, device=proj.device)
+    check(lib().nv_qk_rotate_store(ptr(proj), ptr(bias), proj.stride(0), q_off, k_off, v_off, ptr(q_norm), ptr(k_norm),
+                                   int(q_norm is not None), None, ptr(positions), 0.0, 0, ptr(inv_freq), int(rot_dims),
+                                   float(mscale), ptr(v_first), v_first.stride(0) if v_first is not None else 0,
+                                   ptr(vmix) if v_first is not None else None, scale, eps, ptr(slot_mapping), ptr(cache),
+                                   ptr(q), T, heads, kv_heads, dim, vdim, _code32(cache.dtype), stream()),
+          "nv_qk_rotate_store")
+    return q
+
+
 def qk_store(proj, offsets, positions, scale, slot_mapping, cache, heads, kv_heads, dim, bias=None, temp_coef=0.0,
              temp_every=0):
     """fp32 projections [T, *] with q | k at ``offsets`` (plus ``bias`` over the same columns) -> fp32 queries
@@ -838,10 +879,11 @@ def qk_store(proj, offsets, positions, scale, slot_mapping, cache, heads, kv_hea
 
 def paged_softmax_attn(q, cache, block_tables, cu_q, past_lens, seq_of_token, max_q, heads, kv_heads, dim, vdim, block_size,
                        out, window=0, softcap=0.0, out_scale=1.0, distance_term=False, values_are_keys=False, sink=None,
-                       gate=None):
+                       gate=None, chunk=0, gate_per_head=False):
     """window_attn with its options spelled out: no distance term unless asked for, cache rows that hold keys only and
     serve as values too, a sink logit per head in the denominator, a sigmoid gate (fp32 logits laid out like the
-    output) folded into the store."""
+    output, or with ``gate_per_head`` one per head) folded into the store, and ``chunk`` > 0: a query sees the keys
+    of its own chunk of the sequence only."""
     require_gpu(q, "paged_softmax_attn")
     T = q.size(0)
     assert q.dtype == torch.float32 and q.is_contiguous() and q.size(1) == heads * dim and cache.is_contiguous()
@@ -851,17 +893,17 @@ def paged_softmax_attn(q, cache, block_tables, cu_q, past_lens, seq_of_token, ma
     assert out.dtype == cache.dtype and out.stride(1) == 1 and out.size(0) == T and out.size(1) >= heads * vdim
     assert sink is None or (sink.dtype == cache.dtype and sink.numel() == heads and sink.is_contiguous())
     assert gate is None or (gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.size(0) == T
-                            and gate.size(1) >= heads * vdim)
+                            and gate.size(1) >= (heads if gate_per_head else heads * vdim))
     # steps of one token per request: room for the shares of several workgroups per token (sized before graph capture
     # by the warm-up run of the same shape)
     nbytes = lib().nv_paged_softmax_attn_workspace_bytes(T, max_q, heads, kv_heads, vdim) if cache.dtype == torch.bfloat16 else 0
     ws = workspace(nbytes, q.device, "paged_softmax_attn") if nbytes else None
     check(lib().nv_paged_softmax_attn(ptr(q), ptr(cache), ptr(block_tables), block_tables.size(1), ptr(cu_q),
                                       ptr(past_lens), ptr(seq_of_token), ptr(out), out.stride(0), T, max_q, heads, kv_heads,
-                                      dim, vdim, block_size, window, float(softcap or 0.0), out_scale, int(distance_term),
-                                      int(values_are_keys), ptr(sink), ptr(gate),
-                                      gate.stride(0) if gate is not None else 0, ptr(ws), nbytes, _code32(cache.dtype),
-                                      stream()),
+                                      dim, vdim, block_size, window, int(chunk), float(softcap or 0.0), out_scale,
+                                      int(distance_term), int(values_are_keys), ptr(sink), ptr(gate),
+                                      gate.stride(0) if gate is not None else 0, int(gate_per_head), ptr(ws), nbytes,
+                                      _code32(cache.dtype), stream()),
           "nv_paged_softmax_attn")
     return out
 
@@ -869,7 +911,8 @@ def paged_softmax_attn(q, cache, block_tables, cu_q, past_lens, seq_of_token, ma
 def causal_conv(x, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, act=0, want_f32=True, want_t=False,
                 x_bias=None):
     """Per-channel causal convolution of fp32 rows ``x`` [T, C] (a column slice is fine) with ``w`` [C, taps]; ``state``
-    fp32 [slots, taps - 1, C].  -> (fp32 result or None, result in w's dtype or None)."""
+    fp32 [slots, taps - 1, C].  ``act`` 0: none, 1: SiLU, 2: none, and the token's own input is added (x + conv(x)).
+    -> (fp32 result or None, result in w's dtype or None)."""
     require_gpu(x, "causal_conv")
     T, C = x.shape
     taps = w.size(1)
@@ -926,4 +969,43 @@ def ssd_scan(xbc, z, dt, dt_bias, A_log, D, state, cu_q, past_lens, state_slots,
                             ptr(D), ptr(state), ptr(cu_q), ptr(past_lens), ptr(state_slots), ptr(out), B,
                             heads, groups, state_size, vdim, max_q, ptr(ws), nbytes, _code32(dt_bias.dtype), stream()),
           "nv_ssd_scan")
+    return out
+
+
+def mingru_scan(proj, offsets, z_bias, u_bias, state, cu_q, past_lens, state_slots, channels, out):
+    """Minimal gated recurrent unit over fp32 projections ``proj`` [T, *] with update-gate logits | candidates |
+    output-gate logits at ``offsets`` (``channels`` columns each; the biases of the first two, in out's dtype, are added
+    here); ``state`` fp32 [slots, channels]; ``out`` [T, >= channels] receives S * silu(g)."""
+    require_gpu(proj, "mingru_scan")
+    T = proj.size(0)
+    z_off, u_off, g_off = offsets
+    assert proj.dtype == state.dtype == torch.float32 and proj.stride(1) == 1 and out.stride(1) == 1
+    assert max(z_off, u_off, g_off) + channels <= proj.size(1) and out.size(0) == T and out.size(1) >= channels
+    assert state.is_contiguous() and state.size(-1) == channels
+    for b in (z_bias, u_bias):
+        assert b is None or (b.numel() == channels and b.dtype == out.dtype and b.stride(0) == 1)
+    assert cu_q.dtype == past_lens.dtype == state_slots.dtype == torch.int32
+    check(lib().nv_mingru_scan(ptr(proj), proj.stride(0), z_off, u_off, g_off, ptr(z_bias), ptr(u_bias), ptr(state),
+                               ptr(cu_q), ptr(past_lens), ptr(state_slots), ptr(out), out.stride(0), past_lens.numel(),
+                               channels, _code32(out.dtype), stream()), "nv_mingru_scan")
+    return out
+
+
+def gated_postnorm_add(x, y, w, eps, mult, gate=None, gate_bias=None, out_dtype=None):
+    """fp32 residual rows ``x`` [T, n] += mult * rms_norm(y * sigmoid(gate + gate_bias)) * w, in place (``gate`` None: no
+    gate; ``y`` None: nothing is added); -> the new rows in ``out_dtype`` (None: no copy)."""
+    require_gpu(x, "gated_postnorm_add")
+    T, n = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    if y is not None:
+        assert y.dtype == torch.float32 and y.stride(1) == 1 and y.shape == (T, n) and w.numel() == n and w.is_contiguous()
+        assert gate is None or (gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.shape == (T, n))
+        assert gate_bias is None or (gate_bias.dtype == w.dtype and gate_bias.numel() == n and gate_bias.is_contiguous())
+        assert out_dtype is None or out_dtype == w.dtype
+    out = torch.empty(T, n, dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    code = _code32(out_dtype if out_dtype is not None else w.dtype)
+    check(lib().nv_gated_postnorm_add(ptr(x), ptr(y), y.stride(0) if y is not None else 0, ptr(gate),
+                                      gate.stride(0) if gate is not None else 0, ptr(gate_bias),
+                                      ptr(w) if y is not None else None, ptr(out), n, T, n, eps, mult, code, stream()),
+          "nv_gated_postnorm_add")
     return out

@@ -6,8 +6,10 @@ shared by the heads (the multi-head latent attention of DeepSeek-V2).  Scores of
 
 The up-projections never run over cached tokens: W_uk[h] is folded into the query (q_abs[h] = W_uk[h]^T q_nope[h], one
 small product per head and step token) and W_uv[h] is applied to the attention-weighted sum of latents.  Attention is
-then multi-query attention over rows [c | k_rot] with a sliding window: position i sees j with 0 <= i - j < window.
-Queries go through a latent of their own (RMS-normed), each head's output is multiplied by sigmoid(W_g h)[head].
+then multi-query attention over rows [c | k_rot] with a sliding window: position i sees j with 0 <= i - j < window
+(window 0: every j <= i).  Queries go through a latent of their own (RMS-normed).  The output gate sigmoid(W_g h) has
+one number per head (``gate`` "head") or one per output number (``gate`` "channel", W_g [heads * vdim, width]).  The
+rotated parts turn dimension i with i + dims/2, or with ``interleaved`` dimension 2i with 2i + 1.
 
 A layer built with ``kv_source`` has no key/value down-projection: it reads the cache rows another layer wrote in the
 same step (same kv_rank, rot_dim and rotation), with its own W_uk, W_uv, queries and window.
@@ -27,11 +29,12 @@ from byox_vllm_amd.utils.context import get_context
 class LatentAttention(nn.Module):
     def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, q_rank: int, kv_rank: int, scale: float,
                  window: int, rot_dims: int, rot_base: float, rot_scaling: dict | None, eps: float,
-                 kv_source: "LatentAttention | None" = None):
+                 kv_source: "LatentAttention | None" = None, interleaved: bool = False, gate: str = "head"):
         super().__init__()
         self.heads, self.dim, self.rot_dim, self.vdim = heads, dim, rot_dim, vdim
         self.q_rank, self.kv_rank, self.scale, self.window, self.rot_dims, self.eps = q_rank, kv_rank, scale, window, rot_dims, eps
-        assert rot_dims <= rot_dim and rot_dims % 2 == 0
+        assert rot_dims <= rot_dim and rot_dims % 2 == 0 and gate in ("head", "channel")
+        self.interleaved, self.gate_per_number = bool(interleaved), gate == "channel"
         self.own_kv = kv_source is None
         object.__setattr__(self, "kv_source", kv_source)      # a reference, not a submodule
         if kv_source is not None:
@@ -39,7 +42,7 @@ class LatentAttention(nn.Module):
         shards = {"dq": q_rank}
         if self.own_kv:
             shards["dkv"] = kv_rank + rot_dim
-        shards["g"] = heads
+        shards["g"] = heads * vdim if self.gate_per_number else heads
         self.down = DenseLinear(width, shards=shards)
         self.dq_norm = nn.Parameter(torch.ones(q_rank), requires_grad=False)
         self.uq = DenseLinear(q_rank, heads * (dim + rot_dim))
@@ -67,16 +70,17 @@ class LatentAttention(nn.Module):
         if self.own_kv:
             at = self.down.offset("dkv")
             kernels.latent_kv_store(dn[:, at: at + R + r], self.dkv_norm.data, positions, inv_freq, self.magnitude,
-                                    ctx.slot_mapping, self.cache, R, r, self.rot_dims, self.eps)
+                                    ctx.slot_mapping, self.cache, R, r, self.rot_dims, self.eps, self.interleaved)
         src = self if self.own_kv else self.kv_source
         T = h.size(0)
         qa = torch.empty(T, H * (R + r), dtype=torch.float32, device=h.device)
         kernels.linear(q, self.uk_t.data, out=qa, out_dtype=torch.float32, batch=H, a_batch_stride=d + r,
                        w_batch_stride=R * d, out_batch_stride=R + r, n=R)
-        kernels.latent_q_rope(q, positions, inv_freq, self.magnitude, qa, H, d, r, self.rot_dims, R)
+        kernels.latent_q_rope(q, positions, inv_freq, self.magnitude, qa, H, d, r, self.rot_dims, R, self.interleaved)
         mix = kernels.latent_attn(qa, src.cache, ctx.block_tables, ctx.cu_seqlens_q, ctx.past_lens, ctx.seq_of_token,
                                   H, R, r, src.block_size, self.window, self.scale)
         o = kernels.linear(mix, self.uv.weight.data, batch=H, a_batch_stride=R, w_batch_stride=self.vdim * R,
                            out_batch_stride=self.vdim, n=self.vdim, epilogue=kernels.EPI_ROW_GATE,
+                           act=kernels.GATE_PER_NUMBER if self.gate_per_number else 0,
                            gate=dn[:, self.down.offset("g"):], gate_stride=dn.stride(0))
         return self.o(o, out_dtype=torch.float32)

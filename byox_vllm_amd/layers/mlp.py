@@ -1,5 +1,5 @@
-"""Feed-forward with one up-projection and an element-wise activation, W_down act(W_up h); the activation runs in the
-up-projection's epilogue.  ``xielu`` is the activation with two learned numbers p, q:
+"""Feed-forward with one up-projection and an element-wise activation, W_down act(W_up h) (both products with a bias
+when ``bias``); the activation runs in the up-projection's epilogue.  ``xielu`` is the activation with two learned numbers p, q:
 
     z > 0:  softplus(p) z^2 + z / 2;        z <= 0:  (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2
 
@@ -15,11 +15,11 @@ UNARY = {"silu": kernels.ACT_SILU, "gelu_tanh": kernels.ACT_GELU_TANH, "xielu": 
 
 
 class UnaryMLP(nn.Module):
-    def __init__(self, width: int, ff: int, act: str):
+    def __init__(self, width: int, ff: int, act: str, bias: bool = False):
         super().__init__()
         self.act = UNARY[act]
-        self.up = DenseLinear(width, ff)
-        self.down = DenseLinear(ff, width)
+        self.up = DenseLinear(width, ff, bias=bias)
+        self.down = DenseLinear(ff, width, bias=bias)
         if act == "xielu":
             self.act_params = nn.Parameter(torch.zeros(2, dtype=torch.float32), requires_grad=False)
             self.act_params.weight_loader = lambda p, t: p.data.copy_(t.reshape(2).to(torch.float32))

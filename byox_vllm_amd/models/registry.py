@@ -11,6 +11,7 @@ _MODELS = {
     "Rurutar": ("byox_vllm_amd.models.rurutar", "RurutarForCausalLM"),
     "Nonetar": ("byox_vllm_amd.models.nonetar", "NonetarForCausalLM"),
     "Zamusun": ("byox_vllm_amd.models.zamusun", "ZamusunForCausalLM"),
+    "Kikelorn": ("byox_vllm_amd.models.kikelorn", "KikelornForCausalLM"),
 }
 DEFAULT = "Qwen3ForCausalLM"
 

@@ -340,7 +340,8 @@ int nv_gemm_lt_f32out(const void* x, int64_t x_row_stride, const void* w_rowmajo
  *   epilogue     0 none; 1 gated unit: W holds N gate rows followed by N up rows, out = act(gate) * up with act = SiLU
  *                (act 0) or the tanh form of GELU (act 1), or (act 2) the clamped unit g sigmoid(1.702 g) (u + 1) with
  *                g = min(gate, c), u = clamp(up, -c, c), c = epi_const; 2 soft cap: c * tanh(out / c), c = epi_const;
- *                3 row gate: out *= sigmoid(epi_ptr[m * epi_row_stride + b]);
+ *                3 row gate: out *= sigmoid(epi_ptr[m * epi_row_stride + b]), one logit per row and batch element
+ *                (act 0), or one per output number, epi_ptr[m * epi_row_stride + b * N + n] (act 1);
  *                4 element-wise function chosen by act: 0 SiLU, 1 tanh-form GELU, 2 xIELU (a z^2 + z/2 for z > 0,
  *                b (exp(z) - 1 - z) + z/2 otherwise, with a = epi_ptr[0], b = epi_ptr[1]), 3 out *= epi_const;
  *   out_dtype    NV_BF16 or NV_F32, independent of the operands' dtype. */
@@ -364,6 +365,13 @@ int nv_dyt_norm(float* x, const float* delta, int64_t delta_row_stride, const in
  * projection that re-enters a block of layers with the first residual beside the current one. */
 int nv_residual_pair(float* x, const float* delta, int64_t delta_row_stride, const float* x0, void* out, int64_t rows,
                      int n, int dtype, nv_stream_t stream);
+
+/* Post-norm residual with a gate, on fp32 rows: g = y * sigmoid(gate + gate_bias) (gate null: g = y),
+ * x += mult * g / sqrt(mean(g^2) + eps) * w in place; `out` (may be null) receives the new rows in the storage type.
+ * y null: x is left as it is and only copied to `out`. */
+int nv_gated_postnorm_add(float* x, const float* y, int64_t y_row_stride, const float* gate, int64_t gate_row_stride,
+                          const void* gate_bias, const void* w, void* out, int64_t out_row_stride, int64_t rows, int n,
+                          float eps, float mult, int dtype, nv_stream_t stream);
 
 /* RMS norm of fp32 rows: out = x / sqrt(mean(x^2) + eps) * w, rounded to the storage type. */
 int nv_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* out, int64_t out_row_stride, int64_t rows,
@@ -399,13 +407,15 @@ int nv_matrix_memory(const float* proj, int64_t proj_row_stride, int q_off, int 
                      const int32_t* state_slots, float* out, int64_t out_row_stride, int num_seqs, int heads, int dim,
                      int vdim, int mode, int silu, float q_scale, float cap, int dtype, nv_stream_t stream);
 
-/* Latent attention (csrc/latent_attn.hip): cache rows [kv_rank | rot_dim] per token, shared by all heads. */
+/* Latent attention (csrc/latent_attn.hip): cache rows [kv_rank | rot_dim] per token, shared by all heads.  The first
+ * rot_dims numbers of the rotated parts turn by positions[t] * inv_freq[i]: dimension i with i + rot_dims / 2, or with
+ * `interleaved` dimension 2i with 2i + 1. */
 int nv_latent_kv_store(const float* kv, int64_t kv_row_stride, const void* norm_w, const int64_t* positions,
                        const float* inv_freq, float mscale, const int32_t* slot_mapping, void* cache, int64_t tokens,
-                       int rank, int rot_dim, int rot_dims, float eps, int dtype, nv_stream_t stream);
+                       int rank, int rot_dim, int rot_dims, int interleaved, float eps, int dtype, nv_stream_t stream);
 int nv_latent_q_rope(const void* q, int64_t q_row_stride, const int64_t* positions, const float* inv_freq, float mscale,
-                     float* qa, int64_t tokens, int heads, int dim, int rot_dim, int rot_dims, int rank, int dtype,
-                     nv_stream_t stream);
+                     float* qa, int64_t tokens, int heads, int dim, int rot_dim, int rot_dims, int interleaved, int rank,
+                     int dtype, nv_stream_t stream);
 int nv_latent_attn(const float* qa, const void* cache, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
                    const int32_t* past_lens, const int32_t* seq_of_token, void* out, int64_t tokens, int num_seqs, int heads,
                    int rank,
@@ -466,7 +476,14 @@ int nv_window_attn(const float* q, const void* cache, const int32_t* block_table
  *   1 + temp_coef * ln(floor((positions[t] + 1) / temp_every) + 1).
  * nv_paged_softmax_attn: distance_term 0 drops the distance term; values_are_keys reads rows [k: G * dim] as keys and as
  *   values (vdim == dim); sink [heads] (storage type, may be null) adds exp(sink[h]) to the softmax's denominator; gate
- *   (fp32 [tokens, gate_row_stride], head h at h * vdim, may be null) multiplies the output by its sigmoid. */
+ *   (fp32 [tokens, gate_row_stride], head h at h * vdim, or with gate_per_head one logit per head at column h; may be
+ *   null) multiplies the output by its sigmoid; chunk > 0 restricts a query to the keys of its own chunk,
+ *   floor(i / chunk) == floor(j / chunk), positions counted from the sequence's start.
+ * nv_qk_rotate_store: nv_qk_store with three more options.  norm_whole: one root mean square over all heads * dim query
+ *   numbers (and all kv_heads * dim key numbers), weights [heads * dim] and [kv_heads * dim].  rot_dims > 0: after the
+ *   norm the first rot_dims numbers of every query and key head are rotated, dimension i with i + rot_dims / 2, by the
+ *   angle positions[t] * inv_freq[i], cosine and sine times mscale.  v_first (fp32 [tokens, v_first_row_stride], may be
+ *   null): the stored values are (1 - lam) v + lam v_first with lam = vmix[0] (storage type). */
 int nv_qk_store(const float* proj, const void* bias, int64_t proj_row_stride, int q_off, int k_off, int v_off,
                 const void* q_norm, const void* k_norm, const void* temp, const int64_t* positions, float temp_coef,
                 int temp_every, float scale, float eps, const int32_t* slot_mapping, void* cache, float* q_out,
@@ -474,9 +491,15 @@ int nv_qk_store(const float* proj, const void* bias, int64_t proj_row_stride, in
 int nv_paged_softmax_attn(const float* q, const void* cache, const int32_t* block_tables, int table_cols,
                           const int32_t* cu_q, const int32_t* past_lens, const int32_t* seq_of_token, void* out,
                           int64_t out_row_stride, int64_t tokens, int max_q, int heads, int kv_heads, int dim, int vdim,
-                          int block_size, int window, float softcap, float out_scale, int distance_term,
+                          int block_size, int window, int chunk, float softcap, float out_scale, int distance_term,
                           int values_are_keys, const void* sink, const float* gate, int64_t gate_row_stride,
-                          void* workspace, size_t workspace_bytes, int dtype, nv_stream_t stream);
+                          int gate_per_head, void* workspace, size_t workspace_bytes, int dtype, nv_stream_t stream);
+int nv_qk_rotate_store(const float* proj, const void* bias, int64_t proj_row_stride, int q_off, int k_off, int v_off,
+                       const void* q_norm, const void* k_norm, int norm_whole, const void* temp, const int64_t* positions,
+                       float temp_coef, int temp_every, const float* inv_freq, int rot_dims, float mscale,
+                       const float* v_first, int64_t v_first_row_stride, const void* vmix, float scale, float eps,
+                       const int32_t* slot_mapping, void* cache, float* q_out, int64_t tokens, int heads, int kv_heads,
+                       int dim, int vdim, int dtype, nv_stream_t stream);
 /* Bytes of scratch with which a launch of one token per request (max_q 1) lets several workgroups share a token's
  * keys (their shares are joined by a second kernel); 0 where that does not apply.  Without the scratch (null) the
  * launch keeps one workgroup per token and key/value head. */
@@ -484,7 +507,10 @@ size_t nv_paged_softmax_attn_workspace_bytes(int64_t tokens, int max_q, int head
 
 /* ---- recurrences with an fp32 state per request (csrc/scan.hip) ----
  * nv_causal_conv: per-channel causal convolution over fp32 rows; state [slots, taps - 1, channels] keeps the last
- *   inputs; act 0 none, 1 SiLU; results as fp32 rows and/or rows of the storage type.
+ *   inputs; act 0 none, 1 SiLU, 2 none and the token's own input is added (out = x + conv(x)); results as fp32 rows
+ *   and/or rows of the storage type.
+ * nv_mingru_scan: z = sigmoid(zl + z_bias), u = ul + u_bias, S = (1 - z) S + z c(u) with c(u) = u + 1/2 for u >= 0 and
+ *   sigmoid(u) below, out = S * silu(g); zl, ul and g are the columns z_off, u_off, g_off (+ channels) of fp32 rows.
  * nv_rglru_scan: a = exp(-c sigmoid(gr) softplus(lam)), S = a S + sqrt(1 - a^2) sigmoid(gi) u, out = out_scale * S *
  *   gelu_tanh(y); gates hold, per block of block_width channels, the gr logits followed by the gi logits.
  * nv_ssd_scan: per head, S [state, vdim] <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x, dt = softplus(raw +
@@ -497,6 +523,10 @@ int nv_rglru_scan(const float* u, int64_t u_row_stride, const float* gates, int6
                   const void* y_bias, int64_t y_row_stride, const void* lam, float* state, const int32_t* cu_q, const int32_t* past_lens,
                   const int32_t* state_slots, void* out, int64_t out_row_stride, int num_seqs, int channels,
                   int block_width, float c, float out_scale, int dtype, nv_stream_t stream);
+int nv_mingru_scan(const float* proj, int64_t proj_row_stride, int z_off, int u_off, int g_off, const void* z_bias,
+                   const void* u_bias, float* state, const int32_t* cu_q, const int32_t* past_lens,
+                   const int32_t* state_slots, void* out, int64_t out_row_stride, int num_seqs, int channels, int dtype,
+                   nv_stream_t stream);
 int nv_ssd_scan(const float* xbc, int64_t xbc_row_stride, const float* z, int64_t z_row_stride, const float* dt,
                 int64_t dt_row_stride, const void* dt_bias, const void* A_log, const void* D, float* state,
                 const int32_t* cu_q, const int32_t* past_lens, const int32_t* state_slots, float* out, int num_seqs,
