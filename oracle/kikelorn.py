@@ -99,12 +99,12 @@ def attention_mixer(h, W, p, m, eps, shared):
         f, mag = frequencies(rot)
         pos = torch.arange(T)
         q, k = rotate(q, pos, f, mag, int(rot["dims"]), False), rotate(k, pos, f, mag, int(rot["dims"]), False)
-    if m.get("v_mix"):
+    if m.get("v_mix"):          # blended as flat rows of G * dv numbers: the layers may cut them into heads differently
         if "v_first" in shared:
             lam = W[p + "vmix"]
-            v = (1.0 - lam) * v + lam * shared["v_first"]
+            v = ((1.0 - lam) * v.reshape(T, G * dv) + lam * shared["v_first"]).view(T, G, dv)
         else:
-            shared["v_first"] = v
+            shared["v_first"] = v.reshape(T, G * dv)
     size = (m.get("mask") or {}).get("size")
     o = softmax_attention(q, k, v, float(m["scale"]), chunked(T, int(size)) if size else causal(T))
     o = o * torch.sigmoid(h @ W[p + "g"].T)[:, :, None]
@@ -183,3 +183,59 @@ def forward(tokens, W, cfg, trace=None):
         if trace is not None:
             trace.append(x)
     return (rms(x, eps) * W["final.norm"]) @ W["embed"].T
+
+
+def random_weights(cfg, seed=0):
+    """A checkpoint of the design's tensor names for ``cfg``, values representable in bfloat16."""
+    g = torch.Generator().manual_seed(seed)
+    width, W = cfg["width"], {}
+    taps = int((cfg.get("canon") or {}).get("taps", 0))
+
+    def mat(n, k, s=None):
+        s = (k ** -0.5) if s is None else s
+        return (torch.randn(n, k, generator=g) * s).to(torch.bfloat16)
+
+    def vec(n, s=0.1, at=0.0):
+        return (at + torch.randn(n, generator=g) * s).to(torch.bfloat16)
+
+    W["embed"] = mat(cfg["vocab"], width, 1.0)
+    for i, spec in enumerate(cfg["layers"]):
+        m, p = spec["mixer"], f"l{i}."
+        subs = ("1", "2") if spec.get("mlp") else ("1",)
+        for s in subs:
+            W[p + "norm" + s] = vec(width, 0.2, 1.0)
+            W[p + "rg" + s], W[p + "rg" + s + ".b"] = mat(width, width), vec(width, 0.5)
+            if taps:
+                W[p + "canon" + s] = mat(width, taps, 0.4)
+        if spec["type"] == "attention":
+            H, G, d, dv = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["vdim"]
+            for name, n in (("q", H * d), ("k", G * d), ("v", G * dv)):
+                W[p + "mix." + name] = mat(n, width)
+                if m.get("conv"):
+                    W[p + "mix." + name + ".conv"] = mat(n, m["conv"], 0.6)
+            W[p + "mix.q.norm"], W[p + "mix.k.norm"] = vec(H * d, 0.3, 1.5), vec(G * d, 0.3, 1.5)
+            if m.get("v_mix"):
+                W[p + "mix.vmix"] = (torch.rand((), generator=g) * 0.6 + 0.2).to(torch.bfloat16)
+            W[p + "mix.g"] = mat(H, width)
+            W[p + "mix.o"] = mat(width, H * dv)
+        elif spec["type"] == "latent_attention":
+            H, d, r, dv = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
+            W[p + "mix.dq"], W[p + "mix.dq.norm"] = mat(m["q_rank"], width), vec(m["q_rank"], 0.2, 1.0)
+            W[p + "mix.uq"] = mat(H * (d + r), m["q_rank"], 1.5 * m["q_rank"] ** -0.5)
+            W[p + "mix.dkv"], W[p + "mix.dkv.norm"] = mat(m["kv_rank"] + r, width), vec(m["kv_rank"], 0.2, 1.0)
+            W[p + "mix.uk"] = mat(H * d, m["kv_rank"], 1.5 * m["kv_rank"] ** -0.5)
+            W[p + "mix.uv"] = mat(H * dv, m["kv_rank"])
+            W[p + "mix.g"] = mat(H * dv, width)
+            W[p + "mix.o"] = mat(width, H * dv)
+        else:
+            C = m["width"]
+            W[p + "mix.z"], W[p + "mix.z.b"] = mat(C, width, 2.0 * width ** -0.5), vec(C, 1.0)
+            W[p + "mix.x"], W[p + "mix.x.b"] = mat(C, width), vec(C, 0.5)
+            W[p + "mix.g"] = mat(C, width)
+            W[p + "mix.o"] = mat(width, C)
+        if spec.get("mlp"):
+            ff = spec["mlp"]["ff"]
+            W[p + "mlp.up"], W[p + "mlp.up.b"] = mat(ff, width), vec(ff, 0.3)
+            W[p + "mlp.down"], W[p + "mlp.down.b"] = mat(width, ff), vec(width, 0.3)
+    W["final.norm"] = vec(width, 0.2, 1.0)
+    return W
