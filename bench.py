@@ -282,7 +282,7 @@ def run_generate_workload(args):
     print(json.dumps(line), flush=True)
 
 
-# --arch-compare: the Rurutar, Nonetar and Zamusun designs beside the dense Qwen3 decoder (and beside each other) at equal
+# --arch-compare: the Rurutar, Nonetar, Zamusun and Kikelorn designs beside the dense Qwen3 decoder (and beside each other) at equal
 # width, depth, active feed-forward size and vocabulary, both through LLM.generate: prefill and decode tokens/s.
 # name: (width, layers, prompts, prompt length, decoded tokens)
 ARCH_COMPARE_SIZES = {
@@ -367,13 +367,38 @@ def zamusun_bench_config(width: int, layers: int, vocab: int = 32000):
     return zamusun_config(raw, dtype=torch.bfloat16)
 
 
+def kikelorn_bench_config(width: int, layers: int, vocab: int = 32000):
+    """A Kikelorn configuration with the proportions of a real model's layers, in turn: attention inside chunks of 512
+    tokens (two query heads per key head of 128, four taps behind the projections, half of each head rotated, values
+    shared from the first such layer on), latent attention over the whole context (96 + 32 numbers per query head, a
+    latent of a quarter of the width), and a minimal gated recurrent unit as wide as the model; three input taps in
+    front of every sublayer; feed-forwards of two matrices with the parameter count of the dense comparator's three."""
+    from byox_vllm_amd.models.kikelorn import kikelorn_config
+    heads = width // 128
+    kinds = [
+        {"type": "attention", "mixer": {"heads": heads, "kv_heads": max(1, heads // 2), "dim": 128, "vdim": 128, "conv": 4,
+                                        "mask": {"size": 512}, "rot": {"base": 10000.0, "dims": 64}, "scale": 128 ** -0.5,
+                                        "v_mix": True}},
+        {"type": "latent_attention",
+         "mixer": {"heads": heads, "dim": 96, "rot_dim": 32, "vdim": 128, "kv_rank": width // 4, "q_rank": width // 2,
+                   "scale": 128 ** -0.5, "rot": {"base": 10000.0, "dims": 32,
+                                                 "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}},
+        {"type": "mingru", "mixer": {"width": width}},
+    ]
+    specs = [dict(json.loads(json.dumps(kinds[i % 3])), mlp={"kind": "dense", "ff": 9 * width // 2}) for i in range(layers)]
+    raw = {"architecture": "Kikelorn", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
+           "residual_mult": 0.5, "canon": {"taps": 3}, "layers": specs}
+    return kikelorn_config(raw, dtype=torch.bfloat16)
+
+
 def run_arch_compare(args):
     from byox_vllm_amd import LLM, SamplingParams
     from byox_vllm_amd.config import qwen2_config
     assert args.gpus == 1, "--arch-compare runs on one GPU"
     random.seed(0)
     results = []
-    designs = {"rurutar": rurutar_bench_config, "nonetar": nonetar_bench_config, "zamusun": zamusun_bench_config}
+    designs = {"rurutar": rurutar_bench_config, "nonetar": nonetar_bench_config, "zamusun": zamusun_bench_config,
+               "kikelorn": kikelorn_bench_config}
     chosen = [d for d in args.arch_designs.split(",") if d]
     assert chosen and all(d in designs for d in chosen), f"--arch-designs: a subset of {sorted(designs)}"
     for name, (width, layers, num, plen, decoded) in ARCH_COMPARE_SIZES.items():
@@ -498,7 +523,7 @@ def main():
                     help="instead of the decode benchmark: prefill and decode tokens/s of the designs named by --arch-designs "
                          "beside the dense Qwen3 decoder at equal size (one GPU, LLM.generate)")
     ap.add_argument("--arch-designs", default="rurutar",
-                    help="--arch-compare: the designs to run beside the dense decoder, comma-separated (rurutar, nonetar, zamusun)")
+                    help="--arch-compare: the designs to run beside the dense decoder, comma-separated (rurutar, nonetar, zamusun, kikelorn)")
     ap.add_argument("--arch-sizes", default="", help="--arch-compare: comma-separated subset of " + ",".join(ARCH_COMPARE_SIZES))
     args = ap.parse_args()
     if args.arch_compare:

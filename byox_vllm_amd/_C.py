@@ -70,7 +70,8 @@ _PROTOS = {
                        _i64, _f, _i, _p]),
     "nv_embed_scale": (_i, [_p, _p, _p, _i64, _i, _i64, _f, _i, _p]),
     "nv_dyt_norm": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
-    "nv_gated_postnorm_add": (_i, [_p, _p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i, _f, _f, _i, _p]),
+    "nv_gated_postnorm_add": (_i, [_p, _p, _i64, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i, _f, _f, _i, _p]),
+    "nv_bias_act_f32": (_i, [_p, _p, _i, _p, _i64, _i, _p, _f, _i, _p]),
     "nv_rmsnorm_f32": (_i, [_p, _i64, _p, _p, _i64, _i64, _i, _f, _i, _p]),
     "nv_act_mul_f32": (_i, [_p, _p, _i64, _i, _i, _f, _i, _p]),
     "nv_act_f32": (_i, [_p, _p, _i64, _i, _p, _f, _i, _p]),
@@ -83,6 +84,11 @@ _PROTOS = {
     "nv_latent_kv_store": (_i, [_p, _i64, _p, _p, _p, _f, _p, _p, _i64, _i, _i, _i, _i, _f, _i, _p]),
     "nv_latent_q_rope": (_i, [_p, _i64, _p, _p, _f, _p, _i64, _i, _i, _i, _i, _i, _i, _i, _p]),
     "nv_latent_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _i, _f, _i, _p]),
+    "nv_latent_attn_split": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _i, _f, _i, _p, _sz, _i, _p]),
+    "nv_latent_attn_workspace_bytes": (_sz, [_i64, _i, _i, _i]),
+    "nv_latent_q_rows": (_i, [_p, _i64, _p, _p, _f, _p, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p]),
+    "nv_latent_gather": (_i, [_p, _p, _i, _p, _p, _p, _i, _i, _i, _p, _i64, _i, _p]),
+    "nv_latent_expand": (_i, [_p, _p, _p, _i64, _i, _i, _i, _i, _i, _i, _p]),
     "nv_moe_route": (_i, [_p, _i64, _p, _p, _i64, _i, _i, _i, _p]),
     "nv_moe_sort": (_i, [_p, _i64, _i, _i, _p, _p, _p, _p]),
     "nv_moe_combine": (_i, [_p, _p, _p, _i, _p, _p, _i64, _p, _i64, _i, _p]),

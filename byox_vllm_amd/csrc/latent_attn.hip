@@ -7,6 +7,9 @@
 //   nv_latent_kv_store : RMS norm of the latent, rotation of the shared key part, store into the token's cache row
 //   nv_latent_q_rope   : rotation of the per-head query parts into the absorbed-query buffer
 //   nv_latent_attn     : sliding-window softmax attention, one workgroup per (token, group of heads)
+//   nv_latent_gather, nv_latent_expand, nv_latent_q_rows : the pieces of the EXPANDED form that long prompt portions
+//                        take: the step's requests' cache rows gathered in order, keys and values of every head written
+//                        out from their up-projections, whole query rows; ordinary paged attention reads the result
 //
 // Rotation: dimension i pairs with i + dims/2 ("rotate half"), or with `interleaved` dimension 2i with 2i + 1; the angle
 // is position * inv_freq[i] in fp32, and both cosine and sine are multiplied by `mscale` (the caller folds frequency
@@ -56,10 +59,16 @@ __global__ __launch_bounds__(256) void latent_q_rope_kernel(const T* __restrict_
                                                             const int64_t* __restrict__ positions,
                                                             const float* __restrict__ inv_freq, float mscale,
                                                             float* __restrict__ qa, int H, int dim, int rot_dim,
-                                                            int rot_dims, int rank, int interleaved) {
+                                                            int rot_dims, int rank, int interleaved, int copy_front,
+                                                            float factor) {
   const int64_t t = blockIdx.x;
   const float pos = (float)positions[t];
   const int half = rot_dims / 2;
+  if (copy_front)          // the unrotated numbers in front of the rotated ones (rank == dim): a whole query row
+    for (int idx = threadIdx.x; idx < H * dim; idx += blockDim.x) {
+      const int h = idx / dim, j = idx % dim;
+      qa[(t * H + h) * (rank + rot_dim) + j] = ld_f32<T>(q + t * q_rs + (int64_t)h * (dim + rot_dim) + j) * factor;
+    }
   for (int idx = threadIdx.x; idx < H * rot_dim; idx += blockDim.x) {
     const int h = idx / rot_dim, j = idx % rot_dim;
     const T* src = q + t * q_rs + (int64_t)h * (dim + rot_dim) + dim;
@@ -72,8 +81,50 @@ __global__ __launch_bounds__(256) void latent_q_rope_kernel(const T* __restrict_
       const float other = ld_f32<T>(src + (interleaved ? j ^ 1 : (first ? j + half : j - half)));
       v = first ? v * cs - other * sn : v * cs + other * sn;
     }
-    qa[(t * H + h) * (rank + rot_dim) + rank + j] = v;
+    qa[(t * H + h) * (rank + rot_dim) + rank + j] = v * factor;
   }
+}
+
+// The cache rows of every request of a step, in order of position, into one buffer: request b's row j goes to row
+// cu_k[b] + j (cu_k: starts padded to whole blocks; rows past the request's end are zero).
+template <typename T>
+__global__ __launch_bounds__(256) void latent_gather_kernel(const T* __restrict__ cache, const int32_t* __restrict__ tables,
+                                                            int table_cols, const int32_t* __restrict__ cu_k,
+                                                            const int32_t* __restrict__ cu_q,
+                                                            const int32_t* __restrict__ past, int B, int block_size,
+                                                            int Dk, T* __restrict__ out) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= cu_k[B]) return;
+  const int lane = threadIdx.x & 63;
+  int b = 0;
+  while (b + 1 < B && row >= cu_k[b + 1]) ++b;
+  const int j = (int)(row - cu_k[b]);
+  const int len = past[b] + cu_q[b + 1] - cu_q[b];
+  T* dst = out + row * Dk;
+  if (j >= len) {
+    for (int e = lane; e < Dk; e += 64) dst[e] = (T)0.0f;
+    return;
+  }
+  const T* src = cache + ((int64_t)tables[(int64_t)b * table_cols + j / block_size] * block_size + j % block_size) * Dk;
+  for (int e = lane; e < Dk; e += 64) dst[e] = src[e];
+}
+
+// Expanded key/value rows [k: H * (dim + rot_dim) | v: H * vdim] from the up-projections kv [rows, H * dim | H * vdim]
+// and the gathered cache rows c [rows, rank + rot_dim]: head h's key is [W_uk[h] c | the shared rotated part].
+template <typename T>
+__global__ __launch_bounds__(256) void latent_expand_kernel(const T* __restrict__ kv, const T* __restrict__ c,
+                                                            T* __restrict__ out, int H, int dim, int rot_dim, int vdim,
+                                                            int rank) {
+  const int64_t row = blockIdx.x;
+  const int dk = dim + rot_dim, kw = H * dk, vw = H * vdim;
+  const T* kvr = kv + row * (H * dim + vw);
+  const T* rot = c + row * (rank + rot_dim) + rank;
+  T* dst = out + row * (kw + vw);
+  for (int i = threadIdx.x; i < kw; i += blockDim.x) {
+    const int h = i / dk, e = i % dk;
+    dst[i] = e < dim ? kvr[h * dim + e] : rot[e - dim];
+  }
+  for (int i = threadIdx.x; i < vw; i += blockDim.x) dst[kw + i] = kvr[H * dim + i];
 }
 
 struct AttnArgs {
@@ -189,6 +240,8 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(AttnArgs p) {
 struct MfmaAttnArgs {
   AttnArgs a;
   int B, HQ, TQ, Dkp;
+  int ksplit;              // workgroups that share a tile's keys (blockIdx.z), each walking every ksplit-th key tile;
+  float* partial;          // > 1: their unnormalised shares go to [tokens, H, ksplit, rank + 2] (then maximum and sum)
 };
 
 template <int NTILE, int KEYS>
@@ -274,8 +327,9 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
       }
     }
   };
-  fetch_tile(kmin);
-  for (int j0 = kmin; j0 <= kmax; j0 += ATT_KEYS) {
+  const int kstep = q.ksplit * ATT_KEYS;
+  fetch_tile(kmin + (int)blockIdx.z * ATT_KEYS);
+  for (int j0 = kmin + (int)blockIdx.z * ATT_KEYS; j0 <= kmax; j0 += kstep) {
 #pragma unroll
     for (int u = 0; u < NCH; ++u) {
       const int i = tid + u * 256;
@@ -290,7 +344,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
       }
     }
     __syncthreads();
-    if (j0 + ATT_KEYS <= kmax) fetch_tile(j0 + ATT_KEYS);
+    if (j0 + kstep <= kmax) fetch_tile(j0 + kstep);
     // S = Q K^T: with 64 keys wavefront w takes keys 16 w ..; with 32 keys the wavefront pairs (0, 1) and (2, 3) take
     // the two halves of the feature dimension and their partial scores are summed in the softmax step
     {
@@ -369,6 +423,30 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
     __syncthreads();
   }
   bf16_t* out = reinterpret_cast<bf16_t*>(p.out);
+  if (q.ksplit > 1) {          // another launch joins the shares
+    const int PW = R + 2;
+#pragma unroll
+    for (int n = 0; n < NTILE; ++n) {
+      const int col = 16 * (wv * NTILE + n) + c;
+      if (col >= R) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = 4 * g + r;
+        const int tq = row / q.HQ, hh = h0 + row % q.HQ;
+        if (tq < tcount && hh < p.H)
+          q.partial[(((int64_t)(tstart + tq) * p.H + hh) * q.ksplit + blockIdx.z) * PW + col] = O[n][r];
+      }
+    }
+    if (tid < 16) {
+      const int tq = tid / q.HQ, hh = h0 + tid % q.HQ;
+      if (tq < tcount && hh < p.H) {
+        float* dst = q.partial + (((int64_t)(tstart + tq) * p.H + hh) * q.ksplit + blockIdx.z) * PW + R;
+        dst[0] = sm[tid];
+        dst[1] = sl[tid];
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int n = 0; n < NTILE; ++n) {
     const int col = 16 * (wv * NTILE + n) + c;
@@ -379,6 +457,30 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
       const int tq = row / q.HQ, hh = h0 + row % q.HQ;
       if (tq < tcount && hh < p.H) out[((int64_t)(tstart + tq) * p.H + hh) * R + col] = (bf16_t)(O[n][r] / sl[row]);
     }
+  }
+}
+
+// joins the shares of the ksplit workgroups that walked one (token, head)'s keys: one wavefront per row
+__global__ __launch_bounds__(256) void latent_attn_join_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
+                                                               int64_t rows, int ksplit, int R) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63, PW = R + 2;
+  const float* src = partial + row * ksplit * PW;
+  float m = -INFINITY;
+  for (int z = 0; z < ksplit; ++z) m = fmaxf(m, src[z * PW + R]);
+  float l = 0.0f;
+  for (int z = 0; z < ksplit; ++z) {
+    const float mz = src[z * PW + R];
+    l += mz == -INFINITY ? 0.0f : src[z * PW + R + 1] * __expf(mz - m);
+  }
+  for (int e = lane; e < R; e += 64) {
+    float o = 0.0f;
+    for (int z = 0; z < ksplit; ++z) {
+      const float mz = src[z * PW + R];
+      if (mz != -INFINITY) o += src[z * PW + e] * __expf(mz - m);
+    }
+    out[row * R + e] = (bf16_t)(o / l);
   }
 }
 
@@ -416,22 +518,54 @@ extern "C" int nv_latent_kv_store(const float* kv, int64_t kv_row_stride, const 
 extern "C" int nv_latent_q_rope(const void* q, int64_t q_row_stride, const int64_t* positions, const float* inv_freq,
                                 float mscale, float* qa, int64_t tokens, int heads, int dim, int rot_dim, int rot_dims,
                                 int interleaved, int rank, int dtype, nv_stream_t stream) {
+  return nv_latent_q_rows(q, q_row_stride, positions, inv_freq, mscale, qa, tokens, heads, dim, rot_dim, rot_dims,
+                          interleaved, rank, 0, 1.0f, dtype, stream);
+}
+
+extern "C" int nv_latent_q_rows(const void* q, int64_t q_row_stride, const int64_t* positions, const float* inv_freq,
+                                float mscale, float* qa, int64_t tokens, int heads, int dim, int rot_dim, int rot_dims,
+                                int interleaved, int rank, int copy_front, float factor, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(!copy_front || rank == dim, "nv_latent_q_rows: whole query rows have the unrotated numbers in front");
   NV_CHECK_ARG(q && positions && inv_freq && qa, "nv_latent_q_rope: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_latent_q_rope: bad dtype %d", dtype);
   NV_CHECK_ARG(tokens >= 0 && heads > 0 && dim >= 0 && rot_dim >= 0 && rot_dims <= rot_dim && rot_dims % 2 == 0 && rank > 0,
                "nv_latent_q_rope: bad shape");
-  if (tokens == 0 || rot_dim == 0) return NV_OK;
+  if (tokens == 0 || (rot_dim == 0 && !copy_front)) return NV_OK;
   NV_DISPATCH_T(dtype, latent_q_rope_kernel<T><<<dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream>>>(
                            (const T*)q, q_row_stride, positions, inv_freq, mscale, qa, heads, dim, rot_dim, rot_dims, rank,
-                           interleaved));
+                           interleaved, copy_front, factor));
   NV_CHECK_LAUNCH();
   return NV_OK;
+}
+
+// Workgroups that share one decoded token's keys: enough to put about 256 workgroups on the chip, at most 32.  A
+// function of the launch shape alone (not of the contexts), so a captured launch stays valid as contexts grow.
+static int latent_attn_key_splits(int64_t tokens, int heads) {
+  const int64_t groups = tokens * ((heads + 15) / 16);
+  int k = 1;
+  while (k < 32 && groups * k * 2 <= 512) k *= 2;
+  return k;
+}
+
+extern "C" size_t nv_latent_attn_workspace_bytes(int64_t tokens, int max_q, int heads, int rank) {
+  if (max_q != 1 || tokens <= 0) return 0;
+  const int k = latent_attn_key_splits(tokens, heads);
+  return k > 1 ? (size_t)tokens * heads * k * (rank + 2) * sizeof(float) : 0;
 }
 
 extern "C" int nv_latent_attn(const float* qa, const void* cache, const int32_t* block_tables, int table_cols,
                               const int32_t* cu_q, const int32_t* past_lens, const int32_t* seq_of_token, void* out,
                               int64_t tokens, int num_seqs, int heads, int rank, int rot_dim, int block_size, int window, float scale,
                               int dtype, nv_stream_t stream) {
+  return nv_latent_attn_split(qa, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, tokens, num_seqs,
+                              heads, rank, rot_dim, block_size, window, scale, 0, nullptr, 0, dtype, stream);
+}
+
+extern "C" int nv_latent_attn_split(const float* qa, const void* cache, const int32_t* block_tables, int table_cols,
+                                    const int32_t* cu_q, const int32_t* past_lens, const int32_t* seq_of_token, void* out,
+                                    int64_t tokens, int num_seqs, int heads, int rank, int rot_dim, int block_size,
+                                    int window, float scale, int max_q, void* workspace, size_t workspace_bytes, int dtype,
+                                    nv_stream_t stream) {
   NV_CHECK_ARG(qa && cache && block_tables && cu_q && past_lens && seq_of_token && out, "nv_latent_attn: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_latent_attn: bad dtype %d", dtype);
   NV_CHECK_ARG(tokens >= 0 && tokens <= 65535 * 1024 && heads > 0 && rank > 0 && rot_dim >= 0 && block_size > 0 && table_cols > 0,
@@ -445,7 +579,12 @@ extern "C" int nv_latent_attn(const float* qa, const void* cache, const int32_t*
     while (HQ < heads && HQ < 16) HQ *= 2;
     MfmaAttnArgs q{{qa, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, heads, rank, rot_dim,
                     block_size, window, 0, 0, scale},
-                   num_seqs, HQ, 16 / HQ, ((Dk + 31) / 32) * 32};
+                   num_seqs, HQ, 16 / HQ, ((Dk + 31) / 32) * 32, 1, reinterpret_cast<float*>(workspace)};
+    // one token per request: several workgroups share its keys, when the caller brought room for their shares
+    if (max_q == 1 && workspace) {
+      const int k = latent_attn_key_splits(tokens, heads);
+      if (k > 1 && workspace_bytes >= (size_t)tokens * heads * k * (rank + 2) * sizeof(float)) q.ksplit = k;
+    }
     const int Dq = q.Dkp + 8;
     auto lds_for = [&](int keys) {
       return (size_t)(2 * 16 * Dq + keys * Dq + rank * (keys + 8) + 2 * 16 * (keys + 8)) * 2 + (size_t)(2 * 16 * (keys + 4) + 48) * 4;
@@ -455,7 +594,7 @@ extern "C" int nv_latent_attn(const float* qa, const void* cache, const int32_t*
     if (lds <= 150 * 1024 && keys * (Dk / 8) <= 10 * 256) {
       const int64_t tiles = tokens / q.TQ + num_seqs;        // at most: every request may end in a partial tile
       NV_CHECK_ARG(tiles <= 65535, "nv_latent_attn: %lld tiles exceed one launch", (long long)tiles);
-      dim3 grid((unsigned)((heads + HQ - 1) / HQ), (unsigned)tiles);
+      dim3 grid((unsigned)((heads + HQ - 1) / HQ), (unsigned)tiles, (unsigned)q.ksplit);
       const int ntile = (rank / 16 + 3) / 4;
       hipStream_t st = (hipStream_t)stream;
       hipError_t e;
@@ -469,6 +608,12 @@ extern "C" int nv_latent_attn(const float* qa, const void* cache, const int32_t*
         return NV_ERR_LAUNCH;
       }
       NV_CHECK_LAUNCH();
+      if (q.ksplit > 1) {
+        const int64_t rows = tokens * heads;
+        latent_attn_join_kernel<<<dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st>>>(
+            q.partial, reinterpret_cast<bf16_t*>(out), rows, q.ksplit, rank);
+        NV_CHECK_LAUNCH();
+      }
       return NV_OK;
     }
   }
@@ -485,6 +630,32 @@ extern "C" int nv_latent_attn(const float* qa, const void* cache, const int32_t*
              window, HC, TK, scale};
   dim3 grid((unsigned)((heads + HC - 1) / HC), (unsigned)tokens);
   NV_DISPATCH_T(dtype, latent_attn_kernel<T><<<grid, dim3(256), need(HC, TK), (hipStream_t)stream>>>(p));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_latent_gather(const void* cache, const int32_t* block_tables, int table_cols, const int32_t* cu_k,
+                                const int32_t* cu_q, const int32_t* past_lens, int num_seqs, int block_size, int row_width,
+                                void* out, int64_t rows, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(cache && block_tables && cu_k && cu_q && past_lens && out, "nv_latent_gather: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_latent_gather: bad dtype %d", dtype);
+  NV_CHECK_ARG(num_seqs > 0 && block_size > 0 && row_width > 0 && rows >= 0 && table_cols > 0, "nv_latent_gather: bad shape");
+  if (rows == 0) return NV_OK;
+  NV_DISPATCH_T(dtype, latent_gather_kernel<T><<<dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream>>>(
+                           (const T*)cache, block_tables, table_cols, cu_k, cu_q, past_lens, num_seqs, block_size,
+                           row_width, (T*)out));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_latent_expand(const void* kv, const void* c, void* out, int64_t rows, int heads, int dim, int rot_dim,
+                                int vdim, int rank, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(kv && c && out, "nv_latent_expand: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_latent_expand: bad dtype %d", dtype);
+  NV_CHECK_ARG(rows >= 0 && heads > 0 && dim > 0 && rot_dim >= 0 && vdim > 0 && rank > 0, "nv_latent_expand: bad shape");
+  if (rows == 0) return NV_OK;
+  NV_DISPATCH_T(dtype, latent_expand_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
+                           (const T*)kv, (const T*)c, (T*)out, heads, dim, rot_dim, vdim, rank));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

@@ -51,15 +51,16 @@ __global__ __launch_bounds__(256) void rmsnorm_f32_kernel(const float* __restric
   for (int j = threadIdx.x; j < n; j += blockDim.x) st_f32<T>(out + r * out_rs + j, xr[j] * inv * ld_f32<T>(w + j));
 }
 
-// Post-norm residual with a gate: x[t] += mult * (g / sqrt(mean(g^2) + eps)) * w, g = y[t] * sigmoid(gate[t] + gate_bias)
-// (no gate: g = y); the new row is also written in the storage type for the products that read the residual.  Without y
-// the row is only copied.
+// Post-norm residual with a gate: x[t] += mult * (g / sqrt(mean(g^2) + eps)) * w, g = (y[t] + y_bias) * sigmoid(gate[t] +
+// gate_bias) (no gate: g = y + y_bias; y_bias is the bias a producing product left to its consumer, or null); the new
+// row is also written in the storage type for the products that read the residual.  Without y the row is only copied.
 template <typename T>
 __global__ __launch_bounds__(256) void gated_postnorm_add_kernel(float* __restrict__ x, const float* __restrict__ y,
                                                                  int64_t y_rs, const float* __restrict__ gate,
                                                                  int64_t gate_rs, const T* __restrict__ gate_bias,
-                                                                 const T* __restrict__ w, T* __restrict__ out_t,
-                                                                 int64_t out_rs, int n, float eps, float mult) {
+                                                                 const T* __restrict__ y_bias, const T* __restrict__ w,
+                                                                 T* __restrict__ out_t, int64_t out_rs, int n, float eps,
+                                                                 float mult) {
   __shared__ float red[32];
   const int64_t t = blockIdx.x;
   float* xr = x + t * n;
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(256) void gated_postnorm_add_kernel(float* __restri
   const float* yr = y + t * y_rs;
   const float* gr = gate ? gate + t * gate_rs : nullptr;
   auto gated = [&](int j) {
-    float v = yr[j];
+    float v = yr[j] + (y_bias ? ld_f32<T>(y_bias + j) : 0.0f);
     if (gr) v *= sigmoid_f32(gr[j] + (gate_bias ? ld_f32<T>(gate_bias + j) : 0.0f));
     return v;
   };
@@ -121,10 +122,11 @@ __global__ __launch_bounds__(256) void act_mul_f32_kernel(const float* __restric
 // out = f(y): the element-wise epilogue of nv_linear applied to a plain product's fp32 result (same function codes)
 template <typename T>
 __global__ __launch_bounds__(256) void act_f32_kernel(const float* __restrict__ y, T* __restrict__ out, int64_t total,
-                                                      int act, const float* __restrict__ prm, float c) {
+                                                      int act, const float* __restrict__ prm, float c,
+                                                      const T* __restrict__ bias, int n) {
   const float a = act == 2 ? prm[0] : 0.0f, b = act == 2 ? prm[1] : 0.0f;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
-    const float v = y[i];
+    const float v = y[i] + (bias ? ld_f32<T>(bias + i % n) : 0.0f);
     float r;
     switch (act) {
       case 0: r = silu_f32(v); break;
@@ -228,14 +230,19 @@ extern "C" int nv_act_mul_f32(const float* y, void* out, int64_t rows, int n, in
 
 extern "C" int nv_act_f32(const float* y, void* out, int64_t total, int act, const float* params, float c, int dtype,
                           nv_stream_t stream) {
-  NV_CHECK_ARG(y && out, "nv_act_f32: null pointer");
+  return nv_bias_act_f32(y, nullptr, 1, out, total, act, params, c, dtype, stream);
+}
+
+extern "C" int nv_bias_act_f32(const float* y, const void* bias, int n, void* out, int64_t total, int act,
+                               const float* params, float c, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(y && out && n > 0, "nv_act_f32: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_act_f32: bad dtype %d", dtype);
   NV_CHECK_ARG(total >= 0 && act >= 0 && act <= 3 && (act != 2 || params), "nv_act_f32: bad shape or activation");
   if (total == 0) return NV_OK;
   int64_t blocks = (total + 255) / 256;
   if (blocks > 16384) blocks = 16384;
   NV_DISPATCH_T(dtype, act_f32_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
-                           y, (T*)out, total, act, params, c));
+                           y, (T*)out, total, act, params, c, (const T*)bias, n));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }
@@ -277,7 +284,7 @@ extern "C" int nv_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* 
   return NV_OK;
 }
 
-extern "C" int nv_gated_postnorm_add(float* x, const float* y, int64_t y_row_stride, const float* gate,
+extern "C" int nv_gated_postnorm_add(float* x, const float* y, int64_t y_row_stride, const void* y_bias, const float* gate,
                                      int64_t gate_row_stride, const void* gate_bias, const void* w, void* out,
                                      int64_t out_row_stride, int64_t rows, int n, float eps, float mult, int dtype,
                                      nv_stream_t stream) {
@@ -287,7 +294,7 @@ extern "C" int nv_gated_postnorm_add(float* x, const float* y, int64_t y_row_str
   NV_CHECK_ARG(rows >= 0 && n > 0, "nv_gated_postnorm_add: bad shape");
   if (rows == 0) return NV_OK;
   NV_DISPATCH_T(dtype, gated_postnorm_add_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
-                           x, y, y_row_stride, gate, gate_row_stride, (const T*)gate_bias, (const T*)w, (T*)out,
+                           x, y, y_row_stride, gate, gate_row_stride, (const T*)gate_bias, (const T*)y_bias, (const T*)w, (T*)out,
                            out_row_stride, n, eps, mult));
   NV_CHECK_LAUNCH();
   return NV_OK;

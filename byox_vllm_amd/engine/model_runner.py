@@ -654,10 +654,14 @@ class ModelRunner:
         else:
             rows = [cu[i] + o for i, offsets in enumerate(want) for o in offsets]
         to = lambda data, dt: self._to_device(torch.tensor(data, dtype=dt, device="cpu"))  # noqa: E731
+        cu_context = [0]          # each request's whole context, padded to whole blocks, in one buffer
+        for seq, count in plan:
+            cu_context.append(cu_context[-1] + -(-(seq.num_computed_tokens + count) // bs) * bs)
         set_context(True, cu_seqlens_q=to(cu, torch.int32), max_seqlen_q=max(c for _, c in plan),
                     slot_mapping=to(slots, torch.int32), block_tables=self._prepare_block_tables([s for s, _ in plan]),
                     past_lens=to(past, torch.int32), state_slots=to(state_slots, torch.int32),
-                    seq_of_token=to(seq_of, torch.int32))
+                    seq_of_token=to(seq_of, torch.int32), cu_context=to(cu_context, torch.int32),
+                    context_rows=cu_context[-1])
         try:
             state = self.model(to(ids, torch.int64), to(pos, torch.int64))
             if not rows:

@@ -462,7 +462,8 @@ def linear(x, w, bias=None, out=None, out_dtype=None, *, rows=None, a_rows=None,
     M = x.size(0) if rows is None else rows
     # prefill-sized plain products of a 16-bit model go where the engine sends its other many-row products: the vendor
     # library, here with the result left in fp32
-    if (epilogue in (EPI_NONE, EPI_GLU, EPI_ACT) and batch == 1 and group_offsets is None and a_rows is None and bias is None and out is None
+    if (epilogue in (EPI_NONE, EPI_GLU, EPI_ACT) and batch == 1 and group_offsets is None and a_rows is None
+            and (bias is None or epilogue == EPI_ACT) and out is None
             and rows is None and x.dtype == torch.bfloat16 and (out_dtype or x.dtype) in (torch.float32, torch.bfloat16)
             and w.dim() == 2 and w.is_contiguous() and x.stride(0) % 8 == 0 and use_many_rows_path(M, K, n) and K % 8 == 0
             and n % 8 == 0 and x.data_ptr() % 16 == 0):
@@ -474,7 +475,9 @@ def linear(x, w, bias=None, out=None, out_dtype=None, *, rows=None, a_rows=None,
         if epilogue == EPI_ACT:      # the element-wise function in one pass over the library's fp32 result
             y = _linear_many_rows(x, w, M, n, K, torch.float32)
             out = torch.empty(M, n, dtype=out_dtype or x.dtype, device=x.device)
-            check(lib().nv_act_f32(ptr(y), ptr(out), M * n, act, ptr(gate), cap, _code32(out.dtype), stream()), "nv_act_f32")
+            assert bias is None or (bias.dtype == x.dtype and bias.numel() == n and bias.is_contiguous())
+            check(lib().nv_bias_act_f32(ptr(y), ptr(bias), n, ptr(out), M * n, act, ptr(gate), cap, _code32(out.dtype),
+                                        stream()), "nv_bias_act_f32")
             return out
         return _linear_many_rows(x, w, M, n, K, out_dtype or x.dtype)
     grid_rows = M if group_offsets is None else (max_group_rows if max_group_rows is not None else M)
@@ -658,20 +661,57 @@ def latent_q_rope(q, positions, inv_freq, mscale, qa, heads, dim, rot_dim, rot_d
           "nv_latent_q_rope")
 
 
+def latent_q_rows(q, positions, inv_freq, mscale, heads, dim, rot_dim, rot_dims, factor, interleaved=False):
+    """q [T, heads * (dim + rot_dim)] -> fp32 rows of the same layout, the rotated part turned, everything times
+    ``factor``."""
+    require_gpu(q, "latent_q_rows")
+    assert q.stride(1) == 1 and q.size(1) == heads * (dim + rot_dim) and positions.dtype == torch.int64
+    out = torch.empty(q.size(0), heads * (dim + rot_dim), dtype=torch.float32, device=q.device)
+    check(lib().nv_latent_q_rows(ptr(q), q.stride(0), ptr(positions), ptr(inv_freq), mscale, ptr(out), q.size(0), heads,
+                                 dim, rot_dim, rot_dims, int(interleaved), dim, 1, factor, _code32(q.dtype), stream()),
+          "nv_latent_q_rows")
+    return out
+
+
+def latent_expand(cache, block_tables, cu_k, cu_q, past_lens, block_size, rows, up_weight, heads, dim, rot_dim, vdim, rank):
+    """The expanded keys and values of every request of a step: its cache rows [rank | rot_dim] gathered in order of
+    position (request b at rows cu_k[b] .., padded to whole blocks; ``rows`` = cu_k[-1] on the host), multiplied by
+    ``up_weight`` [heads * dim + heads * vdim, rank] -> [rows, heads * (dim + rot_dim) | heads * vdim] in the cache
+    dtype, laid out like the rows of ordinary paged attention."""
+    require_gpu(cache, "latent_expand")
+    Dk = rank + rot_dim
+    assert cache.is_contiguous() and cache.size(-1) == Dk and up_weight.shape == (heads * (dim + vdim), rank)
+    assert block_tables.dtype == cu_k.dtype == cu_q.dtype == past_lens.dtype == torch.int32 and block_tables.is_contiguous()
+    c = torch.empty(rows, Dk, dtype=cache.dtype, device=cache.device)
+    check(lib().nv_latent_gather(ptr(cache), ptr(block_tables), block_tables.size(1), ptr(cu_k), ptr(cu_q), ptr(past_lens),
+                                 past_lens.numel(), block_size, Dk, ptr(c), rows, _code32(cache.dtype), stream()),
+          "nv_latent_gather")
+    kv = linear(c[:, :rank], up_weight)
+    out = torch.empty(rows, heads * (dim + rot_dim + vdim), dtype=cache.dtype, device=cache.device)
+    check(lib().nv_latent_expand(ptr(kv), ptr(c), ptr(out), rows, heads, dim, rot_dim, vdim, rank, _code32(cache.dtype),
+                                 stream()), "nv_latent_expand")
+    return out
+
+
 def latent_attn(qa, cache, block_tables, cu_q, past_lens, seq_of_token, heads, rank, rot_dim, block_size, window, scale,
-                out=None):
+                out=None, max_q=0):
     """Sliding-window attention of absorbed queries ``qa`` fp32 [T, heads, rank + rot_dim] over the paged latent cache
-    -> [T, heads * rank] in the cache dtype (sum of softmax weights times latents)."""
+    -> [T, heads * rank] in the cache dtype (sum of softmax weights times latents).  ``max_q`` 1 says that every request
+    brings one token: several workgroups may then share a token's keys."""
     require_gpu(qa, "latent_attn")
     T = qa.size(0)
     assert qa.dtype == torch.float32 and qa.is_contiguous() and cache.is_contiguous()
     assert block_tables.dtype == torch.int32 and block_tables.is_contiguous() and block_tables.dim() == 2
     assert cu_q.dtype == past_lens.dtype == seq_of_token.dtype == torch.int32 and seq_of_token.numel() == T
     out = torch.empty(T, heads * rank, dtype=cache.dtype, device=qa.device) if out is None else out
-    check(lib().nv_latent_attn(ptr(qa), ptr(cache), ptr(block_tables), block_tables.size(1), ptr(cu_q), ptr(past_lens),
-                               ptr(seq_of_token), ptr(out), T, past_lens.numel(), heads, rank, rot_dim, block_size, window,
-                               scale,
-                               _code32(cache.dtype), stream()), "nv_latent_attn")
+    # steps of one token per request: room for the shares of several workgroups per token (sized before graph capture
+    # by the warm-up run of the same shape)
+    nbytes = lib().nv_latent_attn_workspace_bytes(T, max_q, heads, rank) if cache.dtype == torch.bfloat16 else 0
+    ws = workspace(nbytes, qa.device, "latent_attn") if nbytes else None
+    check(lib().nv_latent_attn_split(ptr(qa), ptr(cache), ptr(block_tables), block_tables.size(1), ptr(cu_q),
+                                     ptr(past_lens), ptr(seq_of_token), ptr(out), T, past_lens.numel(), heads, rank,
+                                     rot_dim, block_size, window, scale, int(max_q), ptr(ws), nbytes,
+                                     _code32(cache.dtype), stream()), "nv_latent_attn_split")
     return out
 
 
@@ -991,20 +1031,22 @@ def mingru_scan(proj, offsets, z_bias, u_bias, state, cu_q, past_lens, state_slo
     return out
 
 
-def gated_postnorm_add(x, y, w, eps, mult, gate=None, gate_bias=None, out_dtype=None):
-    """fp32 residual rows ``x`` [T, n] += mult * rms_norm(y * sigmoid(gate + gate_bias)) * w, in place (``gate`` None: no
-    gate; ``y`` None: nothing is added); -> the new rows in ``out_dtype`` (None: no copy)."""
+def gated_postnorm_add(x, y, w, eps, mult, gate=None, gate_bias=None, out_dtype=None, y_bias=None):
+    """fp32 residual rows ``x`` [T, n] += mult * rms_norm((y + y_bias) * sigmoid(gate + gate_bias)) * w, in place
+    (``gate`` None: no gate; ``y`` None: nothing is added); -> the new rows in ``out_dtype`` (None: no copy)."""
     require_gpu(x, "gated_postnorm_add")
     T, n = x.shape
     assert x.dtype == torch.float32 and x.is_contiguous()
     if y is not None:
         assert y.dtype == torch.float32 and y.stride(1) == 1 and y.shape == (T, n) and w.numel() == n and w.is_contiguous()
         assert gate is None or (gate.dtype == torch.float32 and gate.stride(1) == 1 and gate.shape == (T, n))
-        assert gate_bias is None or (gate_bias.dtype == w.dtype and gate_bias.numel() == n and gate_bias.is_contiguous())
+        for b in (gate_bias, y_bias):
+            assert b is None or (b.dtype == w.dtype and b.numel() == n and b.is_contiguous())
         assert out_dtype is None or out_dtype == w.dtype
     out = torch.empty(T, n, dtype=out_dtype, device=x.device) if out_dtype is not None else None
     code = _code32(out_dtype if out_dtype is not None else w.dtype)
-    check(lib().nv_gated_postnorm_add(ptr(x), ptr(y), y.stride(0) if y is not None else 0, ptr(gate),
+    check(lib().nv_gated_postnorm_add(ptr(x), ptr(y), y.stride(0) if y is not None else 0,
+                                      ptr(y_bias) if y is not None else None, ptr(gate),
                                       gate.stride(0) if gate is not None else 0, ptr(gate_bias),
                                       ptr(w) if y is not None else None, ptr(out), n, T, n, eps, mult, code, stream()),
           "nv_gated_postnorm_add")

@@ -73,14 +73,51 @@ class LatentAttention(nn.Module):
                                     ctx.slot_mapping, self.cache, R, r, self.rot_dims, self.eps, self.interleaved)
         src = self if self.own_kv else self.kv_source
         T = h.size(0)
+        if self._expands(ctx, h):
+            return self.o(self._expanded(ctx, src, q, dn, positions, inv_freq), out_dtype=torch.float32)
         qa = torch.empty(T, H * (R + r), dtype=torch.float32, device=h.device)
         kernels.linear(q, self.uk_t.data, out=qa, out_dtype=torch.float32, batch=H, a_batch_stride=d + r,
                        w_batch_stride=R * d, out_batch_stride=R + r, n=R)
         kernels.latent_q_rope(q, positions, inv_freq, self.magnitude, qa, H, d, r, self.rot_dims, R, self.interleaved)
         mix = kernels.latent_attn(qa, src.cache, ctx.block_tables, ctx.cu_seqlens_q, ctx.past_lens, ctx.seq_of_token,
-                                  H, R, r, src.block_size, self.window, self.scale)
+                                  H, R, r, src.block_size, self.window, self.scale, max_q=ctx.max_seqlen_q)
         o = kernels.linear(mix, self.uv.weight.data, batch=H, a_batch_stride=R, w_batch_stride=self.vdim * R,
                            out_batch_stride=self.vdim, n=self.vdim, epilogue=kernels.EPI_ROW_GATE,
                            act=kernels.GATE_PER_NUMBER if self.gate_per_number else 0,
                            gate=dn[:, self.down.offset("g"):], gate_stride=dn.stride(0))
         return self.o(o, out_dtype=torch.float32)
+
+    # ------------------------------------------------------------------ long prompt portions
+    EXPAND_FROM = 32          # tokens of one request in a step from which the expanded form is taken
+
+    def _expands(self, ctx, h) -> bool:
+        """Steps that bring a long portion write out keys and values of every head for the contexts of the step's
+        requests (one product over the gathered latents) and run ordinary paged attention over them: a tile of keys
+        then serves 64 tokens of a head instead of one token's heads.  16-bit caches with 16-byte-aligned heads only;
+        single tokens and short portions keep the absorbed form, which never up-projects a cached token."""
+        d, r, dv, R = self.dim, self.rot_dim, self.vdim, self.kv_rank
+        return (h.dtype == torch.bfloat16 and ctx.cu_context is not None and ctx.max_seqlen_q >= self.EXPAND_FROM
+                and (d + r) % 8 == 0 and dv % 8 == 0 and d % 8 == 0 and R % 8 == 0 and d + r <= 256 and dv <= 256)
+
+    def _expanded(self, ctx, src, q, dn, positions, inv_freq):
+        H, d, r, dv, R = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
+        if getattr(self, "_up", None) is None:      # [W_uk; W_uv] over the latent, built once
+            self._up = torch.cat([self.uk_t.data.transpose(1, 2).reshape(H * d, R), self.uv.weight.data]).contiguous()
+        bs = src.block_size
+        rows = kernels.latent_expand(src.cache, ctx.block_tables, ctx.cu_context, ctx.cu_seqlens_q, ctx.past_lens, bs,
+                                     ctx.context_rows, self._up, H, d, r, dv, R)
+        B = ctx.past_lens.numel()
+        cols = ctx.context_rows // bs          # at most: one request owns every block
+        tables = (torch.div(ctx.cu_context[:B], bs, rounding_mode="floor")[:, None]
+                  + torch.arange(cols, dtype=torch.int32, device=q.device)[None]).to(torch.int32).contiguous()
+        qf = kernels.latent_q_rows(q, positions, inv_freq, self.magnitude, H, d, r, self.rot_dims, self.scale,
+                                   self.interleaved)
+        out = torch.empty(q.size(0), H * dv, dtype=q.dtype, device=q.device)
+        g = self.down.offset("g")
+        if self.gate_per_number:
+            gate, per_head = dn[:, g:g + H * dv], False
+        else:
+            gate, per_head = dn[:, g:g + H], True
+        kernels.paged_softmax_attn(qf, rows, tables, ctx.cu_seqlens_q, ctx.past_lens, ctx.seq_of_token, ctx.max_seqlen_q,
+                                   H, H, d + r, dv, bs, out, window=self.window, gate=gate, gate_per_head=per_head)
+        return out

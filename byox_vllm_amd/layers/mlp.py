@@ -31,8 +31,13 @@ class UnaryMLP(nn.Module):
             sp = torch.nn.functional.softplus(self.act_params.data.to(torch.float64))
             self.coef = torch.stack([sp[0], 0.5 + sp[1]]).to(torch.float32).contiguous()
 
-    def forward(self, h):
+    def forward(self, h, defer_bias: bool = False):
+        """-> fp32 [T, width]; with ``defer_bias`` -> (the down-projection without its bias, that bias or None): a caller
+        that adds the bias where it consumes the result keeps the product free of an epilogue."""
         if self.act == kernels.ACT_XIELU and self.coef is None:
             self.finalize()
         hidden = self.up(h, epilogue=kernels.EPI_ACT, act=self.act, gate=self.coef)
+        if defer_bias:
+            return kernels.linear(hidden, self.down.weight.data, out_dtype=torch.float32), \
+                (self.down.bias.data if self.down.bias is not None else None)
         return self.down(hidden, out_dtype=torch.float32)

@@ -18,14 +18,16 @@ from byox_vllm_amd.layers.linear import DenseLinear
 
 
 def fold(x: torch.Tensor, pending, out_dtype=None):
-    """Adds a pending sublayer result (y, gate logits or None, its GatedPostNorm) to the fp32 residual ``x`` in place;
+    """Adds a pending sublayer result (y, gate logits or None, its GatedPostNorm[, a bias still to be added to y]) to the
+    fp32 residual ``x`` in place;
     -> the new rows in ``out_dtype`` (None: no copy)."""
     if pending is None:
         return kernels.gated_postnorm_add(x, None, None, 0.0, 0.0, out_dtype=out_dtype) if out_dtype is not None else None
-    y, logits, norm = pending
+    y, logits, norm = pending[:3]
+    y_bias = pending[3] if len(pending) > 3 else None          # a bias the sublayer's last product left to be added here
     return kernels.gated_postnorm_add(x, y, norm.weight.data, norm.eps, norm.mult, gate=logits,
                                       gate_bias=norm.gate.bias.data if norm.gate is not None else None,
-                                      out_dtype=out_dtype)
+                                      out_dtype=out_dtype, y_bias=y_bias)
 
 
 class GatedPostNorm(nn.Module):

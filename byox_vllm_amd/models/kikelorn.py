@@ -93,7 +93,8 @@ class KikelornLayer(nn.Module):
         pending = (y, logits, self.norm1)
         if self.mlp is not None:
             h, logits = self.norm2.begin(x, pending)
-            pending = (self.mlp(h), logits, self.norm2)
+            y, y_bias = self.mlp(h, defer_bias=True)
+            pending = (y, logits, self.norm2, y_bias)
         return pending
 
 

@@ -24,6 +24,10 @@ class Context:
     past_lens: torch.Tensor | None = None
     state_slots: torch.Tensor | None = None
     seq_of_token: torch.Tensor | None = None
+    # ... and, for steps that bring prompt portions, where each request's whole context (the tokens it holds plus this
+    # step's, padded to whole blocks) would start in one buffer of ``context_rows`` rows: [requests + 1]
+    cu_context: torch.Tensor | None = None
+    context_rows: int = 0
 
 
 _CONTEXT = Context()
@@ -35,10 +39,11 @@ def get_context() -> Context:
 
 def set_context(is_prefill, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=0, max_seqlen_k=0,
                 slot_mapping=None, context_lens=None, block_tables=None, past_lens=None, state_slots=None,
-                seq_of_token=None) -> None:
+                seq_of_token=None, cu_context=None, context_rows=0) -> None:
     global _CONTEXT
     _CONTEXT = Context(is_prefill, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                       slot_mapping, context_lens, block_tables, past_lens, state_slots, seq_of_token)
+                       slot_mapping, context_lens, block_tables, past_lens, state_slots, seq_of_token, cu_context,
+                       context_rows)
 
 
 def reset_context() -> None:

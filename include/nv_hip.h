@@ -366,10 +366,11 @@ int nv_dyt_norm(float* x, const float* delta, int64_t delta_row_stride, const in
 int nv_residual_pair(float* x, const float* delta, int64_t delta_row_stride, const float* x0, void* out, int64_t rows,
                      int n, int dtype, nv_stream_t stream);
 
-/* Post-norm residual with a gate, on fp32 rows: g = y * sigmoid(gate + gate_bias) (gate null: g = y),
- * x += mult * g / sqrt(mean(g^2) + eps) * w in place; `out` (may be null) receives the new rows in the storage type.
- * y null: x is left as it is and only copied to `out`. */
-int nv_gated_postnorm_add(float* x, const float* y, int64_t y_row_stride, const float* gate, int64_t gate_row_stride,
+/* Post-norm residual with a gate, on fp32 rows: g = (y + y_bias) * sigmoid(gate + gate_bias) (gate null: g = y + y_bias;
+ * y_bias, a vector in the storage type, may be null), x += mult * g / sqrt(mean(g^2) + eps) * w in place; `out` (may be
+ * null) receives the new rows in the storage type.  y null: x is left as it is and only copied to `out`. */
+int nv_gated_postnorm_add(float* x, const float* y, int64_t y_row_stride, const void* y_bias, const float* gate,
+                          int64_t gate_row_stride,
                           const void* gate_bias, const void* w, void* out, int64_t out_row_stride, int64_t rows, int n,
                           float eps, float mult, int dtype, nv_stream_t stream);
 
@@ -381,6 +382,9 @@ int nv_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* ou
  * epilogue 1, c its limit. */
 /* nv_act_f32: out = f(y) element-wise over fp32 rows of a plain product, f as in nv_linear's epilogue 4. */
 int nv_act_f32(const float* y, void* out, int64_t total, int act, const float* params, float c, int dtype, nv_stream_t stream);
+/* ... of y + bias, bias [n] in the storage type repeating along the rows of n numbers (null: none). */
+int nv_bias_act_f32(const float* y, const void* bias, int n, void* out, int64_t total, int act, const float* params,
+                    float c, int dtype, nv_stream_t stream);
 int nv_act_mul_f32(const float* y, void* out, int64_t rows, int n, int act, float c, int dtype, nv_stream_t stream);
 
 /* Sampler over fp32 logits: temperature 0 -> argmax (lowest index on ties), else Gumbel-max with noise hashed from
@@ -416,6 +420,27 @@ int nv_latent_kv_store(const float* kv, int64_t kv_row_stride, const void* norm_
 int nv_latent_q_rope(const void* q, int64_t q_row_stride, const int64_t* positions, const float* inv_freq, float mscale,
                      float* qa, int64_t tokens, int heads, int dim, int rot_dim, int rot_dims, int interleaved, int rank,
                      int dtype, nv_stream_t stream);
+/* The expanded form for long prompt portions.  nv_latent_q_rows: nv_latent_q_rope that, with copy_front (rank == dim),
+ * also copies the unrotated numbers in front of the rotated ones, everything times `factor`: fp32 query rows
+ * [heads, dim + rot_dim].  nv_latent_gather: row j of request b's cache rows (0 <= j < past_lens[b] + its tokens) to row
+ * cu_k[b] + j of `out` [rows, row_width], zeros up to cu_k[b + 1].  nv_latent_expand: rows [k: heads * (dim + rot_dim) |
+ * v: heads * vdim] from up-projections kv [rows, heads * dim | heads * vdim] and the gathered rows c [rows, rank +
+ * rot_dim], whose rotated part every head's key ends with. */
+int nv_latent_q_rows(const void* q, int64_t q_row_stride, const int64_t* positions, const float* inv_freq, float mscale,
+                     float* qa, int64_t tokens, int heads, int dim, int rot_dim, int rot_dims, int interleaved, int rank,
+                     int copy_front, float factor, int dtype, nv_stream_t stream);
+int nv_latent_gather(const void* cache, const int32_t* block_tables, int table_cols, const int32_t* cu_k,
+                     const int32_t* cu_q, const int32_t* past_lens, int num_seqs, int block_size, int row_width, void* out,
+                     int64_t rows, int dtype, nv_stream_t stream);
+int nv_latent_expand(const void* kv, const void* c, void* out, int64_t rows, int heads, int dim, int rot_dim, int vdim,
+                     int rank, int dtype, nv_stream_t stream);
+/* nv_latent_attn_split: nv_latent_attn for launches of one token per request (max_q 1): with `workspace` of at least
+ * nv_latent_attn_workspace_bytes several workgroups share a token's keys and a second kernel joins their shares. */
+size_t nv_latent_attn_workspace_bytes(int64_t tokens, int max_q, int heads, int rank);
+int nv_latent_attn_split(const float* qa, const void* cache, const int32_t* block_tables, int table_cols,
+                         const int32_t* cu_q, const int32_t* past_lens, const int32_t* seq_of_token, void* out,
+                         int64_t tokens, int num_seqs, int heads, int rank, int rot_dim, int block_size, int window,
+                         float scale, int max_q, void* workspace, size_t workspace_bytes, int dtype, nv_stream_t stream);
 int nv_latent_attn(const float* qa, const void* cache, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
                    const int32_t* past_lens, const int32_t* seq_of_token, void* out, int64_t tokens, int num_seqs, int heads,
                    int rank,
