@@ -71,6 +71,9 @@ _PROTOS = {
     "nv_embed_scale": (_i, [_p, _p, _p, _i64, _i, _i64, _f, _i, _p]),
     "nv_dyt_norm": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
     "nv_gated_postnorm_add": (_i, [_p, _p, _i64, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i, _f, _f, _i, _p]),
+    "nv_gated_postnorm_add_conv_ok": (_i, [_p, _i, _i]),
+    "nv_gated_postnorm_add_conv": (_i, [_p, _p, _i64, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i, _f, _f, _p, _i, _p, _p, _p,
+                                        _p, _i64, _i, _p]),
     "nv_bias_act_f32": (_i, [_p, _p, _i, _p, _i64, _i, _p, _f, _i, _p]),
     "nv_rmsnorm_f32": (_i, [_p, _i64, _p, _p, _i64, _i64, _i, _f, _i, _p]),
     "nv_act_mul_f32": (_i, [_p, _p, _i64, _i, _i, _f, _i, _p]),
@@ -105,6 +108,8 @@ _PROTOS = {
                                 _p, _p, _i64, _i, _i, _i, _i, _i, _p]),
     "nv_paged_softmax_attn_workspace_bytes": (_sz, [_i64, _i, _i, _i, _i]),
     "nv_causal_conv": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _i, _i, _i, _i, _p]),
+    "nv_causal_conv_batch": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _i, _i, _i, _i, _i,
+                                  _p]),
     "nv_rglru_scan": (_i, [_p, _i64, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _i, _f, _f, _i, _p]),
     "nv_mingru_scan": (_i, [_p, _i64, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _i, _p]),
     "nv_ssd_scan": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _sz, _i,

@@ -460,27 +460,29 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
   }
 }
 
-// joins the shares of the ksplit workgroups that walked one (token, head)'s keys: one wavefront per row
+// joins the shares of the ksplit (at most 32) workgroups that walked one (token, head)'s keys: one workgroup per row,
+// the shares' weights exp(m_z - m) / l first, then every thread sums its columns over the shares
 __global__ __launch_bounds__(256) void latent_attn_join_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
-                                                               int64_t rows, int ksplit, int R) {
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
-  const int lane = threadIdx.x & 63, PW = R + 2;
+                                                               int ksplit, int R) {
+  __shared__ float wz[32];
+  const int64_t row = blockIdx.x;
+  const int PW = R + 2;
   const float* src = partial + row * ksplit * PW;
-  float m = -INFINITY;
-  for (int z = 0; z < ksplit; ++z) m = fmaxf(m, src[z * PW + R]);
-  float l = 0.0f;
-  for (int z = 0; z < ksplit; ++z) {
-    const float mz = src[z * PW + R];
-    l += mz == -INFINITY ? 0.0f : src[z * PW + R + 1] * __expf(mz - m);
+  if (threadIdx.x < 64) {
+    const int z = threadIdx.x;
+    const float mz = z < ksplit ? src[z * PW + R] : -INFINITY;
+    const float lz = z < ksplit ? src[z * PW + R + 1] : 0.0f;
+    const float m = wave_max(mz);
+    const float f = mz == -INFINITY ? 0.0f : __expf(mz - m);
+    const float l = wave_sum(lz * f);
+    if (z < 32) wz[z] = f / l;
   }
-  for (int e = lane; e < R; e += 64) {
+  __syncthreads();
+  for (int e = threadIdx.x; e < R; e += 256) {
     float o = 0.0f;
-    for (int z = 0; z < ksplit; ++z) {
-      const float mz = src[z * PW + R];
-      if (mz != -INFINITY) o += src[z * PW + e] * __expf(mz - m);
-    }
-    out[row * R + e] = (bf16_t)(o / l);
+#pragma unroll 8
+    for (int z = 0; z < ksplit; ++z) o += src[z * PW + e] * wz[z];
+    out[row * R + e] = (bf16_t)o;
   }
 }
 
@@ -610,8 +612,8 @@ extern "C" int nv_latent_attn_split(const float* qa, const void* cache, const in
       NV_CHECK_LAUNCH();
       if (q.ksplit > 1) {
         const int64_t rows = tokens * heads;
-        latent_attn_join_kernel<<<dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st>>>(
-            q.partial, reinterpret_cast<bf16_t*>(out), rows, q.ksplit, rank);
+        latent_attn_join_kernel<<<dim3((unsigned)rows), dim3(256), 0, st>>>(q.partial, reinterpret_cast<bf16_t*>(out),
+                                                                            q.ksplit, rank);
         NV_CHECK_LAUNCH();
       }
       return NV_OK;

@@ -54,23 +54,128 @@ __global__ __launch_bounds__(256) void rmsnorm_f32_kernel(const float* __restric
 // Post-norm residual with a gate: x[t] += mult * (g / sqrt(mean(g^2) + eps)) * w, g = (y[t] + y_bias) * sigmoid(gate[t] +
 // gate_bias) (no gate: g = y + y_bias; y_bias is the bias a producing product left to its consumer, or null); the new
 // row is also written in the storage type for the products that read the residual.  Without y the row is only copied.
-template <typename T>
+template <typename T> struct Pack4;
+template <> struct Pack4<float> {
+  typedef f32x4 type;
+  static __device__ __forceinline__ f32x4 widen(const f32x4& v) { return v; }
+  static __device__ __forceinline__ f32x4 narrow(const f32x4& v) { return v; }
+};
+template <> struct Pack4<bf16_t> {
+  typedef uint2 type;
+  static __device__ __forceinline__ f32x4 widen(const uint2& v) {
+    return f32x4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                 __uint_as_float(v.y & 0xffff0000u)};
+  }
+  static __device__ __forceinline__ uint2 narrow(const f32x4& v) {
+    union { bf16_t h[4]; uint2 u; } r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r.h[i] = (bf16_t)v[i];
+    return r.u;
+  }
+};
+
+// The input convolution of the NEXT sublayer, for steps in which row t is request t's only token: every earlier row a
+// tap reads is in the request's slot, so the launch that makes the new residual row also hands out x + conv(x) and moves
+// the slot on (csrc/scan.hip has the general form).
+struct NextConv {
+  const void* w;          // [n, taps], or null: no convolution in this launch
+  float* state;           // [slots, taps - 1, n]
+  const int32_t* slots;   // [rows]
+  const int32_t* past;    // [rows] tokens the request holds already (0: the slot's contents do not count)
+  void* out;              // [rows, out_rs] in the storage type
+  int64_t out_rs;
+  int taps;
+};
+constexpr int NEXT_CONV_MAX_TAPS = 8;
+
+// NV > 0: rows of at most NV * 1024 numbers, a multiple of 4, every pointer 16-byte aligned: a thread keeps its gated
+// values in registers between the two passes and moves four numbers per access.  NV == 0: any row.
+template <typename T, int NV>
 __global__ __launch_bounds__(256) void gated_postnorm_add_kernel(float* __restrict__ x, const float* __restrict__ y,
                                                                  int64_t y_rs, const float* __restrict__ gate,
                                                                  int64_t gate_rs, const T* __restrict__ gate_bias,
                                                                  const T* __restrict__ y_bias, const T* __restrict__ w,
                                                                  T* __restrict__ out_t, int64_t out_rs, int n, float eps,
-                                                                 float mult) {
+                                                                 float mult, NextConv cv) {
   __shared__ float red[32];
+  typedef typename Pack4<T>::type P;
   const int64_t t = blockIdx.x;
   float* xr = x + t * n;
-  if (y == nullptr) {
+  if (y == nullptr && (NV == 0 || cv.w == nullptr)) {
     if (out_t)
       for (int j = threadIdx.x; j < n; j += blockDim.x) st_f32<T>(out_t + t * out_rs + j, xr[j]);
     return;
   }
   const float* yr = y + t * y_rs;
   const float* gr = gate ? gate + t * gate_rs : nullptr;
+  if constexpr (NV > 0) {
+    const int n4 = n >> 2;
+    f32x4 g[NV];
+    float ss = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int c = threadIdx.x + k * 256;
+      g[k] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      if (c < n4 && y) {
+        f32x4 v = reinterpret_cast<const f32x4*>(yr)[c];
+        if (y_bias) {
+          const f32x4 b = Pack4<T>::widen(reinterpret_cast<const P*>(y_bias)[c]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] += b[i];
+        }
+        if (gr) {
+          f32x4 z = reinterpret_cast<const f32x4*>(gr)[c];
+          if (gate_bias) {
+            const f32x4 b = Pack4<T>::widen(reinterpret_cast<const P*>(gate_bias)[c]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) z[i] += b[i];
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] *= sigmoid_f32(z[i]);
+        }
+        g[k] = v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ss += v[i] * v[i];
+      }
+    }
+    if (y) ss = block_sum(ss, red);
+    const float inv = mult / sqrtf(ss / (float)n + eps);
+    const int keep = cv.taps - 1;
+    float* slot = cv.w ? cv.state + (int64_t)cv.slots[t] * keep * n : nullptr;
+    const bool fresh = cv.w && cv.past[t] == 0;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int c = threadIdx.x + k * 256;
+      if (c < n4) {
+        f32x4 v = reinterpret_cast<f32x4*>(xr)[c];
+        if (y) {
+          const f32x4 wv = Pack4<T>::widen(reinterpret_cast<const P*>(w)[c]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] += g[k][i] * inv * wv[i];
+          reinterpret_cast<f32x4*>(xr)[c] = v;
+        }
+        if (out_t) reinterpret_cast<P*>(out_t + t * out_rs)[c] = Pack4<T>::narrow(v);
+        if (cv.w) {
+          // tap j reads the row keep - j tokens back: slot row j for j < keep, the new row for the last tap
+          const T* cw = reinterpret_cast<const T*>(cv.w) + (int64_t)c * 4 * cv.taps;
+          f32x4 h = v;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) h[i] += ld_f32<T>(cw + i * cv.taps + keep) * v[i];
+#pragma unroll
+          for (int j = 0; j < NEXT_CONV_MAX_TAPS - 1; ++j) {
+            if (j >= keep) continue;
+            f32x4 old = fresh ? f32x4{0.0f, 0.0f, 0.0f, 0.0f} : reinterpret_cast<const f32x4*>(slot + (int64_t)j * n)[c];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) h[i] += ld_f32<T>(cw + i * cv.taps + j) * old[i];
+            if (j > 0) reinterpret_cast<f32x4*>(slot + (int64_t)(j - 1) * n)[c] = old;      // the slot moves on by one row
+          }
+          if (keep > 0) reinterpret_cast<f32x4*>(slot + (int64_t)(keep - 1) * n)[c] = v;
+          reinterpret_cast<P*>(reinterpret_cast<T*>(cv.out) + t * cv.out_rs)[c] = Pack4<T>::narrow(h);
+        }
+      }
+    }
+    return;
+  }
   auto gated = [&](int j) {
     float v = yr[j] + (y_bias ? ld_f32<T>(y_bias + j) : 0.0f);
     if (gr) v *= sigmoid_f32(gr[j] + (gate_bias ? ld_f32<T>(gate_bias + j) : 0.0f));
@@ -288,14 +393,43 @@ extern "C" int nv_gated_postnorm_add(float* x, const float* y, int64_t y_row_str
                                      int64_t gate_row_stride, const void* gate_bias, const void* w, void* out,
                                      int64_t out_row_stride, int64_t rows, int n, float eps, float mult, int dtype,
                                      nv_stream_t stream) {
+  return nv_gated_postnorm_add_conv(x, y, y_row_stride, y_bias, gate, gate_row_stride, gate_bias, w, out, out_row_stride,
+                                    rows, n, eps, mult, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0, dtype, stream);
+}
+
+extern "C" int nv_gated_postnorm_add_conv_ok(const void* x, int n, int taps) {
+  return n % 4 == 0 && n <= 4096 && ((uintptr_t)x & 15) == 0 && taps >= 1 && taps <= NEXT_CONV_MAX_TAPS;
+}
+
+extern "C" int nv_gated_postnorm_add_conv(float* x, const float* y, int64_t y_row_stride, const void* y_bias,
+                                          const float* gate, int64_t gate_row_stride, const void* gate_bias, const void* w,
+                                          void* out, int64_t out_row_stride, int64_t rows, int n, float eps, float mult,
+                                          const void* conv_w, int taps, float* conv_state, const int32_t* state_slots,
+                                          const int32_t* past_lens, void* conv_out, int64_t conv_out_row_stride, int dtype,
+                                          nv_stream_t stream) {
   NV_CHECK_ARG(x && (y == nullptr || w), "nv_gated_postnorm_add: null pointer");
-  NV_CHECK_ARG(y || out, "nv_gated_postnorm_add: nothing to do");
+  NV_CHECK_ARG(y || out || conv_w, "nv_gated_postnorm_add: nothing to do");
+  NV_CHECK_ARG(!conv_w || ((conv_state || taps == 1) && state_slots && past_lens && conv_out &&
+                           nv_gated_postnorm_add_conv_ok(x, n, taps)),
+               "nv_gated_postnorm_add: the fused convolution needs its slots, and rows of a multiple of 4 up to 4096");
+  NextConv cv{conv_w, conv_state, state_slots, past_lens, conv_out, conv_out_row_stride, taps};
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_gated_postnorm_add: bad dtype %d", dtype);
   NV_CHECK_ARG(rows >= 0 && n > 0, "nv_gated_postnorm_add: bad shape");
   if (rows == 0) return NV_OK;
-  NV_DISPATCH_T(dtype, gated_postnorm_add_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
-                           x, y, y_row_stride, gate, gate_row_stride, (const T*)gate_bias, (const T*)y_bias, (const T*)w, (T*)out,
-                           out_row_stride, n, eps, mult));
+  auto al16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  const bool vec = (y || conv_w) && n % 4 == 0 && n <= 4096 && al16(x) && al16(y) && al16(gate) && al16(gate_bias) &&
+                   al16(y_bias) && al16(w) && al16(out) && al16(conv_state) && al16(conv_out) && y_row_stride % 4 == 0 &&
+                   gate_row_stride % 4 == 0 && out_row_stride % 4 == 0 && conv_out_row_stride % 4 == 0;
+  NV_CHECK_ARG(vec || !conv_w, "nv_gated_postnorm_add: the fused convolution needs 16-byte aligned rows");
+#define NV_POSTNORM(NVAL)                                                                                              \
+  NV_DISPATCH_T(dtype, gated_postnorm_add_kernel<T, NVAL><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>( \
+                           x, y, y_row_stride, gate, gate_row_stride, (const T*)gate_bias, (const T*)y_bias,           \
+                           (const T*)w, (T*)out, out_row_stride, n, eps, mult, cv))
+  if (vec && n <= 1024) NV_POSTNORM(1);
+  else if (vec && n <= 2048) NV_POSTNORM(2);
+  else if (vec) NV_POSTNORM(4);
+  else NV_POSTNORM(0);
+#undef NV_POSTNORM
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

@@ -34,6 +34,8 @@ struct ConvArgs {
   void* out_t;            // [tokens, ot_rs] in the storage type, or null
   int64_t ot_rs;
   int C, taps, act;       // act 0: none, 1: SiLU, 2: none, and the token's own input is added to the result
+  int heads_only;         // 1: blockIdx.x counts requests; only the tokens that reach back over a portion's start are served
+  int64_t tokens;
 };
 
 // One thread per (token, channel).  Only a portion's first taps - 1 tokens need the slot; they are all served by the
@@ -42,9 +44,10 @@ struct ConvArgs {
 template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs p) {
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
-  const int64_t t = blockIdx.x;
   if (c >= p.C) return;
-  const int b = p.seq_of[t];
+  if (p.heads_only && p.cu_q[blockIdx.x + 1] <= p.cu_q[blockIdx.x]) return;
+  const int64_t t = p.heads_only ? p.cu_q[blockIdx.x] : blockIdx.x;
+  const int b = p.heads_only ? blockIdx.x : p.seq_of[t];
   const int64_t t0 = p.cu_q[b];
   const int k = (int)(t - t0), taps = p.taps, keep = taps - 1;
   if (k > 0 && k < keep) return;
@@ -91,6 +94,74 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs p) {
     if (i >= keep) continue;
     const int src = n - keep + i;
     slot[(int64_t)i * p.C + c] = src >= 0 ? p.x[(t0 + src) * p.x_rs + c] + xb : st[i + n];
+  }
+}
+
+// The tokens that lie at least taps - 1 rows behind their portion's start need no slot: a thread takes four channels
+// and CONV_TT consecutive tokens of the packed batch, keeps the last taps rows in registers and moves 16 bytes per
+// access.  (The others, and the slots, are served by causal_conv_kernel with heads_only.)  C % 4 == 0, aligned rows.
+constexpr int CONV_TT = 8;
+
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_rows_kernel(ConvArgs p) {
+  const int c4 = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c4 * 4 >= p.C) return;
+  const int c = c4 * 4, taps = p.taps, keep = taps - 1;
+  const int64_t t_begin = (int64_t)blockIdx.x * CONV_TT, t_end = min(p.tokens, t_begin + CONV_TT);
+  f32x4 wt[CONV_MAX_TAPS], win[CONV_MAX_TAPS];
+  const T* w = reinterpret_cast<const T*>(p.w);
+#pragma unroll
+  for (int j = 0; j < CONV_MAX_TAPS; ++j)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) wt[j][i] = j < taps ? ld_f32<T>(w + (int64_t)(c + i) * taps + j) : 0.0f;
+  f32x4 bias = f32x4{0.f, 0.f, 0.f, 0.f}, xb = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (p.bias) bias[i] = ld_f32<T>(reinterpret_cast<const T*>(p.bias) + c + i);
+    if (p.x_bias) xb[i] = ld_f32<T>(reinterpret_cast<const T*>(p.x_bias) + c + i);
+  }
+  auto row = [&](int64_t tt) {
+    f32x4 v = *reinterpret_cast<const f32x4*>(p.x + max(tt, (int64_t)0) * p.x_rs + c);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] += xb[i];
+    return v;
+  };
+  // inside the walk win[CONV_MAX_TAPS - 1] is the current token's row and win[CONV_MAX_TAPS - 1 - m] the row m tokens
+  // back; before it the window stands one token earlier
+#pragma unroll
+  for (int i = 0; i < CONV_MAX_TAPS; ++i) {
+    const int back = CONV_MAX_TAPS - i;
+    win[i] = (back >= 1 && back <= keep) ? row(t_begin - back) : f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  for (int64_t tt = t_begin; tt < t_end; ++tt) {
+#pragma unroll
+    for (int i = 0; i + 1 < CONV_MAX_TAPS; ++i) win[i] = win[i + 1];
+    win[CONV_MAX_TAPS - 1] = row(tt);
+    const int b = p.seq_of[tt];
+    if ((int)(tt - p.cu_q[b]) < keep) continue;          // reaches back over its portion's start
+    f32x4 v = bias;
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {            // tap j reads the row keep - j tokens back
+      const int idx = CONV_MAX_TAPS - 1 - (keep - j);
+      if (j < taps && idx >= 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] += wt[j][i] * win[idx][i];
+      }
+    }
+    if (p.act == 1) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = silu_f32(v[i]);
+    }
+    if (p.act == 2) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] += win[CONV_MAX_TAPS - 1][i];
+    }
+    if (p.out_f32) *reinterpret_cast<f32x4*>(p.out_f32 + tt * p.of_rs + c) = v;
+    if (p.out_t) {
+      T* dst = reinterpret_cast<T*>(p.out_t) + tt * p.ot_rs + c;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) st_f32<T>(dst + i, v[i]);
+    }
   }
 }
 
@@ -376,6 +447,15 @@ extern "C" int nv_causal_conv(const float* x, const void* x_bias, int64_t x_row_
                               const int32_t* seq_of_token, float* out_f32, int64_t out_f32_row_stride, void* out_t,
                               int64_t out_t_row_stride, int64_t tokens, int channels, int taps, int act, int dtype,
                               nv_stream_t stream) {
+  return nv_causal_conv_batch(x, x_bias, x_row_stride, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, out_f32,
+                              out_f32_row_stride, out_t, out_t_row_stride, tokens, 0, channels, taps, act, dtype, stream);
+}
+
+extern "C" int nv_causal_conv_batch(const float* x, const void* x_bias, int64_t x_row_stride, const void* w,
+                                    const void* bias, float* state, const int32_t* cu_q, const int32_t* past_lens,
+                                    const int32_t* state_slots, const int32_t* seq_of_token, float* out_f32,
+                                    int64_t out_f32_row_stride, void* out_t, int64_t out_t_row_stride, int64_t tokens,
+                                    int num_seqs, int channels, int taps, int act, int dtype, nv_stream_t stream) {
   NV_CHECK_ARG(x && w && (state || taps == 1) && cu_q && past_lens && state_slots && seq_of_token && (out_f32 || out_t),
                "nv_causal_conv: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_causal_conv: bad dtype %d", dtype);
@@ -384,7 +464,26 @@ extern "C" int nv_causal_conv(const float* x, const void* x_bias, int64_t x_row_
                "nv_causal_conv: bad shape (taps up to %d)", CONV_MAX_TAPS);
   if (tokens == 0) return NV_OK;
   ConvArgs p{x, x_bias, x_row_stride, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, out_f32, out_f32_row_stride,
-             out_t, out_t_row_stride, channels, taps, act};
+             out_t, out_t_row_stride, channels, taps, act, 0, tokens};
+  // with the number of requests known: one launch over the requests for the tokens that need the slot, and (where a
+  // request brings more tokens than that) one over all rows, four channels and several tokens per thread
+  const size_t tsz = dtype == NV_BF16 ? 2 : 4;
+  if (num_seqs > 0 && num_seqs <= 65535 && channels % 4 == 0 && x_row_stride % 4 == 0 && (uintptr_t)x % 16 == 0 &&
+      (!out_f32 || (out_f32_row_stride % 4 == 0 && (uintptr_t)out_f32 % 16 == 0)) &&
+      (!out_t || ((out_t_row_stride * tsz) % 8 == 0 && (uintptr_t)out_t % 8 == 0))) {
+    p.heads_only = 1;
+    NV_DISPATCH_T(dtype, causal_conv_kernel<T><<<dim3((unsigned)num_seqs, (unsigned)((channels + 255) / 256)), dim3(256), 0,
+                                                 (hipStream_t)stream>>>(p));
+    NV_CHECK_LAUNCH();
+    if (tokens > num_seqs) {
+      const int c4 = channels / 4, threads = c4 >= 256 ? 256 : ((c4 + 63) / 64) * 64;
+      NV_DISPATCH_T(dtype, causal_conv_rows_kernel<T><<<dim3((unsigned)((tokens + CONV_TT - 1) / CONV_TT),
+                                                            (unsigned)((c4 + threads - 1) / threads)),
+                                                       dim3(threads), 0, (hipStream_t)stream>>>(p));
+      NV_CHECK_LAUNCH();
+    }
+    return NV_OK;
+  }
   NV_DISPATCH_T(dtype, causal_conv_kernel<T><<<dim3((unsigned)tokens, (unsigned)((channels + 255) / 256)), dim3(256), 0,
                                                (hipStream_t)stream>>>(p));
   NV_CHECK_LAUNCH();

@@ -963,9 +963,10 @@ def causal_conv(x, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, a
     of = torch.empty(T, C, dtype=torch.float32, device=x.device) if want_f32 else None
     ot = torch.empty(T, C, dtype=w.dtype, device=x.device) if want_t else None
     assert x_bias is None or (x_bias.numel() == C and x_bias.dtype == w.dtype and x_bias.stride(0) == 1)
-    check(lib().nv_causal_conv(ptr(x), ptr(x_bias), x.stride(0), ptr(w), ptr(bias), ptr(state), ptr(cu_q), ptr(past_lens),
-                               ptr(state_slots), ptr(seq_of_token), ptr(of), C, ptr(ot), C, T, C, taps, act,
-                               _code32(w.dtype), stream()), "nv_causal_conv")
+    assert cu_q.numel() == past_lens.numel() + 1
+    check(lib().nv_causal_conv_batch(ptr(x), ptr(x_bias), x.stride(0), ptr(w), ptr(bias), ptr(state), ptr(cu_q),
+                                     ptr(past_lens), ptr(state_slots), ptr(seq_of_token), ptr(of), C, ptr(ot), C, T,
+                                     past_lens.numel(), C, taps, act, _code32(w.dtype), stream()), "nv_causal_conv_batch")
     return of, ot
 
 
@@ -1031,9 +1032,11 @@ def mingru_scan(proj, offsets, z_bias, u_bias, state, cu_q, past_lens, state_slo
     return out
 
 
-def gated_postnorm_add(x, y, w, eps, mult, gate=None, gate_bias=None, out_dtype=None, y_bias=None):
+def gated_postnorm_add(x, y, w, eps, mult, gate=None, gate_bias=None, out_dtype=None, y_bias=None, conv=None):
     """fp32 residual rows ``x`` [T, n] += mult * rms_norm((y + y_bias) * sigmoid(gate + gate_bias)) * w, in place
-    (``gate`` None: no gate; ``y`` None: nothing is added); -> the new rows in ``out_dtype`` (None: no copy)."""
+    (``gate`` None: no gate; ``y`` None: nothing is added); -> the new rows in ``out_dtype`` (None: no copy).
+    ``conv`` = (weight [n, taps], state [slots, taps - 1, n], state_slots, past_lens), for steps in which row t is the
+    only token of request t: -> (rows, x + conv(x) in the weight's dtype), the slots moved on by that token."""
     require_gpu(x, "gated_postnorm_add")
     T, n = x.shape
     assert x.dtype == torch.float32 and x.is_contiguous()
@@ -1044,6 +1047,20 @@ def gated_postnorm_add(x, y, w, eps, mult, gate=None, gate_bias=None, out_dtype=
             assert b is None or (b.dtype == w.dtype and b.numel() == n and b.is_contiguous())
         assert out_dtype is None or out_dtype == w.dtype
     out = torch.empty(T, n, dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    if conv is not None:
+        cw, state, slots, past = conv
+        taps = cw.size(1)
+        assert cw.shape == (n, taps) and cw.is_contiguous() and state.is_contiguous() and state.shape[1:] == (taps - 1, n)
+        assert slots.dtype == past.dtype == torch.int32 and slots.numel() == past.numel() == T
+        assert (y is None or cw.dtype == w.dtype) and (out_dtype is None or out_dtype == cw.dtype)
+        hc = torch.empty(T, n, dtype=cw.dtype, device=x.device)
+        check(lib().nv_gated_postnorm_add_conv(ptr(x), ptr(y), y.stride(0) if y is not None else 0,
+                                               ptr(y_bias) if y is not None else None, ptr(gate),
+                                               gate.stride(0) if gate is not None else 0, ptr(gate_bias),
+                                               ptr(w) if y is not None else None, ptr(out), n, T, n, eps, mult, ptr(cw),
+                                               taps, ptr(state), ptr(slots), ptr(past), ptr(hc), n, _code32(cw.dtype),
+                                               stream()), "nv_gated_postnorm_add_conv")
+        return out, hc
     code = _code32(out_dtype if out_dtype is not None else w.dtype)
     check(lib().nv_gated_postnorm_add(ptr(x), ptr(y), y.stride(0) if y is not None else 0,
                                       ptr(y_bias) if y is not None else None, ptr(gate),

@@ -374,6 +374,17 @@ int nv_gated_postnorm_add(float* x, const float* y, int64_t y_row_stride, const 
                           const void* gate_bias, const void* w, void* out, int64_t out_row_stride, int64_t rows, int n,
                           float eps, float mult, int dtype, nv_stream_t stream);
 
+/* ... and, for steps in which row t is the only token of the request with slot state_slots[t], the input convolution of
+ * the next sublayer in the same launch: conv_out = x + conv(x) with conv_w [n, taps], the earlier rows read from, and
+ * the new row pushed into, conv_state [slots, taps - 1, n] (past_lens[t] == 0: the slot's contents do not count).
+ * nv_gated_postnorm_add_conv_ok says whether a row shape can take this form. */
+int nv_gated_postnorm_add_conv_ok(const void* x, int n, int taps);
+int nv_gated_postnorm_add_conv(float* x, const float* y, int64_t y_row_stride, const void* y_bias, const float* gate,
+                               int64_t gate_row_stride, const void* gate_bias, const void* w, void* out,
+                               int64_t out_row_stride, int64_t rows, int n, float eps, float mult, const void* conv_w,
+                               int taps, float* conv_state, const int32_t* state_slots, const int32_t* past_lens,
+                               void* conv_out, int64_t conv_out_row_stride, int dtype, nv_stream_t stream);
+
 /* RMS norm of fp32 rows: out = x / sqrt(mean(x^2) + eps) * w, rounded to the storage type. */
 int nv_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* out, int64_t out_row_stride, int64_t rows,
                    int n, float eps, int dtype, nv_stream_t stream);
@@ -544,6 +555,13 @@ int nv_causal_conv(const float* x, const void* x_bias, int64_t x_row_stride, con
                    const int32_t* cu_q, const int32_t* past_lens, const int32_t* state_slots, const int32_t* seq_of_token,
                    float* out_f32, int64_t out_f32_row_stride, void* out_t, int64_t out_t_row_stride, int64_t tokens,
                    int channels, int taps, int act, int dtype, nv_stream_t stream);
+/* nv_causal_conv with the number of requests of the step (cu_q has num_seqs + 1 entries): lets the launch serve the rows
+ * that need no slot four channels and several tokens per thread.  0: unknown. */
+int nv_causal_conv_batch(const float* x, const void* x_bias, int64_t x_row_stride, const void* w, const void* bias,
+                         float* state, const int32_t* cu_q, const int32_t* past_lens, const int32_t* state_slots,
+                         const int32_t* seq_of_token, float* out_f32, int64_t out_f32_row_stride, void* out_t,
+                         int64_t out_t_row_stride, int64_t tokens, int num_seqs, int channels, int taps, int act, int dtype,
+                         nv_stream_t stream);
 int nv_rglru_scan(const float* u, int64_t u_row_stride, const float* gates, int64_t gates_row_stride, const float* y,
                   const void* y_bias, int64_t y_row_stride, const void* lam, float* state, const int32_t* cu_q, const int32_t* past_lens,
                   const int32_t* state_slots, void* out, int64_t out_row_stride, int num_seqs, int channels,
