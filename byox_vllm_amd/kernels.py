@@ -463,7 +463,7 @@ def linear(x, w, bias=None, out=None, out_dtype=None, *, rows=None, a_rows=None,
     # prefill-sized plain products of a 16-bit model go where the engine sends its other many-row products: the vendor
     # library, here with the result left in fp32
     if (epilogue in (EPI_NONE, EPI_GLU, EPI_ACT) and batch == 1 and group_offsets is None and a_rows is None
-            and (bias is None or epilogue == EPI_ACT) and out is None
+            and (bias is None or (epilogue == EPI_ACT and (out_dtype or x.dtype) == x.dtype)) and out is None
             and rows is None and x.dtype == torch.bfloat16 and (out_dtype or x.dtype) in (torch.float32, torch.bfloat16)
             and w.dim() == 2 and w.is_contiguous() and x.stride(0) % 8 == 0 and use_many_rows_path(M, K, n) and K % 8 == 0
             and n % 8 == 0 and x.data_ptr() % 16 == 0):

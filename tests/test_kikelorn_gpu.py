@@ -51,10 +51,13 @@ def test_gated_postnorm_add(dtype, n, gated):
     logits, bias = torch.randn(9, n + 5, generator=g) * 2, _round(torch.randn(n, generator=g), dtype)
     w = _round(1 + 0.3 * torch.randn(n, generator=g), dtype)
     xd = x.to(DEV)
+    yb = _round(torch.randn(n, generator=g), dtype) if n != 96 else None       # a bias its product left to be added here
     out = kernels.gated_postnorm_add(xd, y.to(DEV)[:, 3:], w.to(DEV).to(dtype), 1e-5, 0.7,
                                      gate=logits.to(DEV)[:, 5:] if gated else None,
-                                     gate_bias=bias.to(DEV).to(dtype) if gated else None, out_dtype=dtype)
-    gy = y[:, 3:].double() * (torch.sigmoid(logits[:, 5:].double() + bias.double()) if gated else 1.0)
+                                     gate_bias=bias.to(DEV).to(dtype) if gated else None, out_dtype=dtype,
+                                     y_bias=yb.to(DEV).to(dtype) if yb is not None else None)
+    gy = y[:, 3:].double() + (yb.double() if yb is not None else 0.0)
+    gy = gy * (torch.sigmoid(logits[:, 5:].double() + bias.double()) if gated else 1.0)
     want = x.double() + 0.7 * O.rms(gy, 1e-5) * w.double()
     _close(xd, want, 1e-6)                                         # the residual itself stays fp32
     assert torch.equal(out.cpu(), xd.cpu().to(dtype))
@@ -75,32 +78,74 @@ def test_postnorm_eps_sits_inside_the_root():
     assert torch.equal(x[0].cpu(), torch.ones(64)) and abs(float(x[1, 0]) - want) < 1e-6
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,taps", [(100, 3), (96, 1), (2048, 4), (1028, 2), (4096, 5)])
+def test_postnorm_launch_runs_the_next_input_convolution_for_single_tokens(dtype, n, taps):
+    """Three requests decode side by side, one joins later in a slot another has left, one sits a step out: the fused
+    launch must give the residual of the plain launch and x + conv(x) of the whole sequences."""
+    from byox_vllm_amd import kernels
+    g = torch.Generator().manual_seed(n + taps)
+    lens = {"a": 9, "b": 4, "c": 7, "d": 5}
+    ys = {k: torch.randn(v, n, generator=g) * 3 for k, v in lens.items()}
+    w = _round(1 + 0.3 * torch.randn(n, generator=g), dtype)
+    cw = _round(torch.randn(n, taps, generator=g) * 0.5, dtype)
+    # the residual of a request: x_t = x0_t + 0.5 * rms(y_t) * w, rows independent of each other
+    x0 = {k: torch.randn(v, n, generator=g) for k, v in lens.items()}
+    xs = {k: x0[k].double() + 0.5 * O.rms(ys[k].double(), 1e-5) * w.double() for k in lens}
+    want = {k: xs[k] + O.causal_conv(xs[k], cw.double()) for k in lens}
+    state = torch.full((4, taps - 1, n), float("nan"), device=DEV)
+    at = {k: 0 for k in lens}
+    slot = {"a": 0, "b": 2, "c": 1}
+    steps = [["a", "b", "c"], ["a", "b"], ["a", "b", "c"], ["b", "c", "a"], ["a", "c", "d"], ["d", "a", "c"], ["c", "d", "a"],
+             ["a", "d", "c"], ["d", "a", "c"], ["a"]]
+    for names in steps:
+        if "d" in names and "d" not in slot:
+            slot["d"] = slot["b"]                     # b is over: its slot is used again
+        names = [k for k in names if at[k] < lens[k]]
+        if not names:
+            continue
+        x = torch.stack([x0[k][at[k]] for k in names]).to(DEV)
+        y = torch.stack([ys[k][at[k]] for k in names]).to(DEV)
+        rows, h = kernels.gated_postnorm_add(x, y, w.to(DEV).to(dtype), 1e-5, 0.5, out_dtype=dtype,
+                                             conv=(cw.to(DEV).to(dtype), state, _i32([slot[k] for k in names]),
+                                                   _i32([at[k] for k in names])))
+        for i, k in enumerate(names):
+            _close(x[i], xs[k][at[k]], 1e-6)
+            _close(h[i].float(), want[k][at[k]], 2e-6 if dtype == torch.float32 else 8e-3)
+            at[k] += 1
+        assert torch.equal(rows, x.to(dtype))
+    assert at == lens and torch.isnan(state[3]).all()
+
+
 # ------------------------------------------------------------------------------------------------ input convolution
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("taps", [1, 2, 3, 5])
 @pytest.mark.parametrize("pieces", PIECES)
-def test_input_convolution_in_pieces(dtype, taps, pieces):
-    """x + conv(x) over one request cut into pieces down to one token, from a slot that held something else."""
+@pytest.mark.parametrize("C", [70, 72])
+def test_input_convolution_in_pieces(dtype, taps, pieces, C):
+    """x + conv(x) over one request cut into pieces down to one token, from a slot that held something else; channel
+    counts that do and do not split into groups of four."""
     from byox_vllm_amd import kernels
-    C, T = 70, 40
+    T = 40
     g = torch.Generator().manual_seed(taps)
-    x = torch.randn(T, C + 2, generator=g)
+    x = torch.randn(T, C + 4, generator=g)
     w = _round(torch.randn(C, taps, generator=g) * 0.5, dtype)
     state = torch.full((3, taps - 1, C), float("nan"), device=DEV)
     xd, wd, outs = x.to(DEV), w.to(DEV).to(dtype), []
     for a, n, cu, past, slots, seq_of in _steps(pieces, slot=2):
-        outs.append(kernels.causal_conv(xd[a:a + n, 2:], wd, None, state, cu, past, slots, seq_of, act=2, want_f32=True,
+        outs.append(kernels.causal_conv(xd[a:a + n, 4:], wd, None, state, cu, past, slots, seq_of, act=2, want_f32=True,
                                         want_t=True))
-    want = x[:, 2:].double() + O.causal_conv(x[:, 2:].double(), w.double())
+    want = x[:, 4:].double() + O.causal_conv(x[:, 4:].double(), w.double())
     _close(torch.cat([o[0] for o in outs]), want, 1e-6)
     assert torch.equal(torch.cat([o[1] for o in outs]), torch.cat([o[0] for o in outs]).to(dtype))
     assert torch.isnan(state[:2]).all() and not torch.isnan(state[2]).any()
 
 
-def test_input_convolution_keeps_requests_apart():
+@pytest.mark.parametrize("C", [33, 64])
+def test_input_convolution_keeps_requests_apart(C):
     """Two requests in one launch, the second continuing from its slot: no tap reaches into the neighbour's rows."""
     from byox_vllm_amd import kernels
-    C, taps = 33, 4
+    taps = 4
     g = torch.Generator().manual_seed(0)
     xa, xb = torch.randn(6, C, generator=g), torch.randn(9, C, generator=g)
     w = torch.randn(C, taps, generator=g)
@@ -380,6 +425,21 @@ def test_per_number_gate_in_the_value_up_projection(dtype, rows, H, R, dv):
     _close(got, want * torch.sigmoid(logits[:, 7:].double()), 2e-5)
 
 
+@pytest.mark.parametrize("rows", [100, 4200])
+def test_up_projection_with_bias_and_gelu(rows):
+    """Few rows take nv_linear's epilogue, thousands the vendor library and one pass over its fp32 result."""
+    from byox_vllm_amd import kernels
+    g = torch.Generator().manual_seed(rows)
+    x = _round(torch.randn(rows, 256, generator=g), torch.bfloat16)
+    w = _round(torch.randn(384, 256, generator=g) / 16, torch.bfloat16)
+    b = _round(torch.randn(384, generator=g), torch.bfloat16)
+    want = O.gelu_tanh(x.double() @ w.double().T + b.double())
+    for out_dtype, tol in ((torch.float32, 2e-5), (torch.bfloat16, 8e-3)):
+        got = kernels.linear(x.to(DEV).bfloat16(), w.to(DEV).bfloat16(), b.to(DEV).bfloat16(), epilogue=kernels.EPI_ACT,
+                             act=kernels.ACT_GELU_TANH, out_dtype=out_dtype)
+        _close(got.float(), want, tol)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("pieces", [[600], [599, 1], [560] + [1] * 40, [300, 300]])
 def test_latent_attention_hears_a_far_key_among_hundreds(dtype, pieces):
@@ -404,7 +464,7 @@ def test_latent_attention_hears_a_far_key_among_hundreds(dtype, pieces):
     outs = []
     for a, n, cu, past, _, seq_of in _steps(pieces):
         outs.append(kernels.latent_attn(qa[a:a + n].contiguous().to(DEV), cache, _i32([pages]), cu, past, seq_of, H, R, r,
-                                        block, 0, 1.0))
+                                        block, 0, 1.0, max_q=n))        # single tokens: their keys split over workgroups
     got = torch.cat(outs).float().view(T, H, R)
     s = torch.einsum("thc,jc->htj", qa.double(), rows.double()).masked_fill(~O.causal(T)[None], float("-inf"))
     want = torch.einsum("htj,jc->thc", torch.softmax(s, -1), rows[:, :R].double())
