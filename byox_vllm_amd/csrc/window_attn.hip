@@ -66,6 +66,17 @@ __global__ __launch_bounds__(256) void qk_norm_store_kernel(QkArgs p) {
   const T* bias = reinterpret_cast<const T*>(p.bias);
   const int half = p.rot_dims / 2;
   const float pos = p.rot_dims > 0 ? (float)p.positions[t] : 0.0f;
+  // cosine and sine of the token's angles once for all heads (rotations over more than 256 numbers evaluate them in place)
+  __shared__ float s_cs[128], s_sn[128];
+  const bool trig_shared = half > 0 && half <= 128;
+  if (trig_shared) {
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+      const float a = pos * p.inv_freq[i];
+      s_cs[i] = cosf(a) * p.mscale;
+      s_sn[i] = sinf(a) * p.mscale;
+    }
+    __syncthreads();
+  }
   float inv_q = 1.0f, inv_k = 1.0f;
   if (qn && p.norm_whole) {
     float sq = 0.0f, sk = 0.0f;
@@ -105,8 +116,16 @@ __global__ __launch_bounds__(256) void qk_norm_store_kernel(QkArgs p) {
       float x = normed(e);
       if (e < p.rot_dims) {
         const bool first = e < half;
-        const float a = pos * p.inv_freq[first ? e : e - half];
-        const float cs = cosf(a) * p.mscale, sn = sinf(a) * p.mscale;
+        const int fi = first ? e : e - half;
+        float cs, sn;
+        if (trig_shared) {
+          cs = s_cs[fi];
+          sn = s_sn[fi];
+        } else {
+          const float a = pos * p.inv_freq[fi];
+          cs = cosf(a) * p.mscale;
+          sn = sinf(a) * p.mscale;
+        }
         const float other = normed(first ? e + half : e - half);
         x = first ? x * cs - other * sn : x * cs + other * sn;
       }
@@ -296,7 +315,8 @@ constexpr size_t ma_lds_bytes(int ks, int ct, bool split) {
   return split ? 4 * (ma_stage_bytes(ks, ct) + 16 * MA_PST * 2) : ma_stage_bytes(ks, ct) + 4 * 16 * MA_PST * 2;
 }
 
-template <int KS, int CT, bool SPLIT>
+// EXT: chunks and the gate of one logit per head are compiled in; launches that use neither take the kernel without them
+template <int KS, int CT, bool SPLIT, bool EXT>
 __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
   constexpr int DK = KS * 32, KST = DK + 8, DVP = CT * 16;
   constexpr int STAGE = (int)(ma_stage_bytes(KS, CT) / 2);                 // bf16 elements of one staging area
@@ -354,7 +374,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
       }
     }
     // the four accumulator rows of this lane
-    int pos[4], kmin[4];      // kmin: first key of the row's chunk
+    int pos[4], kmin[EXT ? 4 : 1];      // kmin: first key of the row's chunk
     float slope[4], m_run[4], l_run[4];
     bool valid[4];
 #pragma unroll
@@ -362,7 +382,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
       const int rr = row0 + lg * 4 + r;
       valid[r] = rr < rows;
       pos[r] = p0 + rr / R;
-      kmin[r] = p.chunk > 0 ? pos[r] / p.chunk * p.chunk : 0;
+      if constexpr (EXT) kmin[r] = p.chunk > 0 ? pos[r] / p.chunk * p.chunk : 0;
       slope[r] = p.slope_on ? exp2f(-8.0f * (float)(g * R + rr % R + 1) / (float)p.H) : 0.0f;
       m_run[r] = -INFINITY;
       l_run[r] = 0.0f;
@@ -372,9 +392,9 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
     for (int ct = 0; ct < CT; ++ct) acc_o[ct] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     const int wpos_lo = p0 + row0 / R, wpos_hi = p0 + min(rows - 1, row0 + 15) / R;
 
-    int lo = p.window > 0 ? max(0, p0 - p.window + 1) : 0;
-    if (p.chunk > 0) lo = max(lo, p0 / p.chunk * p.chunk);      // the tile's first token has the earliest chunk
-    const int hi = p0 + nq - 1;
+    const int lo_w = p.window > 0 ? max(0, p0 - p.window + 1) : 0;
+    // the tile's first token has the earliest chunk
+    const int lo = (EXT && p.chunk > 0) ? max(lo_w, p0 / p.chunk * p.chunk) : lo_w, hi = p0 + nq - 1;
     const int walkers = SPLIT ? 4 * p.ksplit : 1;          // wavefronts (of all workgroups) that share this token's keys
     for (int j0 = lo + (SPLIT ? ((int)blockIdx.z * 4 + wv) * MA_KEYS : 0); j0 <= hi; j0 += walkers * MA_KEYS) {
       if (stid < MA_KEYS) {
@@ -416,8 +436,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
       }
       sync();
       // keys this wavefront's rows can see: [wpos_lo - window + 1, wpos_hi]
-      const bool need = wave_on && j0 <= wpos_hi && (p.window <= 0 || j0 + MA_KEYS - 1 > wpos_lo - p.window) &&
-                        (p.chunk <= 0 || j0 + MA_KEYS - 1 >= wpos_lo / p.chunk * p.chunk);
+      bool need = wave_on && j0 <= wpos_hi && (p.window <= 0 || j0 + MA_KEYS - 1 > wpos_lo - p.window);
+      if constexpr (EXT) need = need && (p.chunk <= 0 || j0 + MA_KEYS - 1 >= wpos_lo / p.chunk * p.chunk);
       if (need) {
         f32x4 acc_s[4];
 #pragma unroll
@@ -440,7 +460,8 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
             float sc = acc_s[sub][r];
             if (p.softcap > 0.0f) sc = p.softcap * tanhf(sc / p.softcap);
             sc -= slope[r] * (float)dist;
-            const bool vis = valid[r] && dist >= 0 && (p.window <= 0 || dist < p.window) && kp >= kmin[r];
+            bool vis = valid[r] && dist >= 0 && (p.window <= 0 || dist < p.window);
+            if constexpr (EXT) vis = vis && kp >= kmin[r];
             sc = vis ? sc : -INFINITY;
             acc_s[sub][r] = sc;
             mt = fmaxf(mt, sc);
@@ -526,7 +547,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
         float f, den;
         close_softmax(m, l, sink != nullptr, sink ? ld_f32<bf16_t>(sink + h) : 0.0f, f, den);
         float v = o * f * p.out_scale / den;
-        if (p.gate) v *= sigmoid_f32(p.gate[(ts + rr / R) * p.gate_rs + (p.gate_head ? h : h * dv + e)]);
+        if (p.gate) v *= sigmoid_f32(p.gate[(ts + rr / R) * p.gate_rs + ((EXT && p.gate_head) ? h : h * dv + e)]);
         out[(ts + rr / R) * p.out_rs + h * dv + e] = (bf16_t)v;
       }
       __syncthreads();
@@ -540,11 +561,11 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
         close_softmax(m_run[r], l_run[r], sink != nullptr, sink ? ld_f32<bf16_t>(sink + h) : 0.0f, fs, den);
         const float f = p.out_scale * fs / den;
         bf16_t* orow = out + (ts + rr / R) * p.out_rs + h * dv;
-        const float* grow = p.gate ? p.gate + (ts + rr / R) * p.gate_rs + (p.gate_head ? h : h * dv) : nullptr;
+        const float* grow = p.gate ? p.gate + (ts + rr / R) * p.gate_rs + ((EXT && p.gate_head) ? h : h * dv) : nullptr;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
           const int e = ct * 16 + lc;
-          if (e < dv) orow[e] = (bf16_t)(acc_o[ct][r] * f * (grow ? sigmoid_f32(grow[p.gate_head ? 0 : e]) : 1.0f));
+          if (e < dv) orow[e] = (bf16_t)(acc_o[ct][r] * f * (grow ? sigmoid_f32(grow[(EXT && p.gate_head) ? 0 : e]) : 1.0f));
         }
       }
     }
@@ -589,18 +610,24 @@ __global__ __launch_bounds__(256) void window_attn_join_kernel(WAttnArgs p) {
   }
 }
 
-template <int KS, int CT, bool SPLIT>
-hipError_t launch_window_mfma3(const WAttnArgs& p, dim3 grid, hipStream_t s) {
+template <int KS, int CT, bool SPLIT, bool EXT>
+hipError_t launch_window_mfma4(const WAttnArgs& p, dim3 grid, hipStream_t s) {
   constexpr size_t lds = ma_lds_bytes(KS, CT, SPLIT);
   static size_t allowed = 64 * 1024;
   if (lds > allowed) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&window_attn_mfma_kernel<KS, CT, SPLIT>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&window_attn_mfma_kernel<KS, CT, SPLIT, EXT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     allowed = lds;
   }
-  window_attn_mfma_kernel<KS, CT, SPLIT><<<grid, dim3(256), lds, s>>>(p);
+  window_attn_mfma_kernel<KS, CT, SPLIT, EXT><<<grid, dim3(256), lds, s>>>(p);
   return hipGetLastError();
+}
+
+template <int KS, int CT, bool SPLIT>
+hipError_t launch_window_mfma3(const WAttnArgs& p, dim3 grid, hipStream_t s) {
+  if (p.chunk > 0 || (p.gate && p.gate_head)) return launch_window_mfma4<KS, CT, SPLIT, true>(p, grid, s);
+  return launch_window_mfma4<KS, CT, SPLIT, false>(p, grid, s);
 }
 
 template <int KS, int CT>
