@@ -387,7 +387,7 @@ def kikelorn_bench_config(width: int, layers: int, vocab: int = 32000):
     ]
     specs = [dict(json.loads(json.dumps(kinds[i % 3])), mlp={"kind": "dense", "ff": 9 * width // 2}) for i in range(layers)]
     raw = {"architecture": "Kikelorn", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
-           "residual_mult": 0.5, "canon": {"taps": 3}, "layers": specs}
+           "residual_mult": 0.7, "canon": {"taps": 3}, "layers": specs}
     return kikelorn_config(raw, dtype=torch.bfloat16)
 
 

@@ -40,7 +40,7 @@ def dense(ff):
     return {"kind": "dense", "ff": ff}
 
 
-def config(vocab, width, layers, taps=3, mult=0.5, scale=1.0, eps=1e-5):
+def config(vocab, width, layers, taps=2, mult=0.8, scale=1.0, eps=1e-5):
     cfg = {"architecture": "Kikelorn", "vocab": vocab, "width": width, "norm": {"eps": eps}, "residual_mult": mult,
            "embedding": {"scale": scale}, "layers": [dict(copy.deepcopy(mixer), mlp=mlp) for mixer, mlp in layers]}
     if taps:
@@ -80,7 +80,7 @@ def aligned_config():
         (latent(4, 32, 16, 32, 48, 64, 48 ** -0.5, base=50000.0, scaling=(4.0, 32, 8.0, 1.0)), dense(128)),
         (mingru(128), dense(64)),
         (attention(4, 4, 64, 16, 0.125, chunk=40, rot=(1000.0, 64), v_mix=True), None),
-    ], taps=2, mult=0.5, scale=2.0)
+    ], taps=2, mult=0.6, scale=2.0)
 
 
 def plain_config():

@@ -177,7 +177,7 @@ def _mingru_run(proj, offs, C, zb, ub, pieces, state, slot, dtype=torch.float32,
     return torch.cat(outs).float()
 
 
-@pytest.mark.parametrize("C", [70, 64, 224, 1])
+@pytest.mark.parametrize("C", [70, 64, 200, 1])
 @pytest.mark.parametrize("pieces", PIECES + [[16, 16, 8], [3, 37]])
 def test_mingru_in_pieces(C, pieces):
     g = torch.Generator().manual_seed(C)
