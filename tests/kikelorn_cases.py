@@ -93,6 +93,42 @@ def plain_config():
     ], taps=0, mult=0.25, scale=1.25)
 
 
+def random_config(seed: int):
+    """A configuration drawn from a seed: three to six layers of any kind in any order, head counts, sizes, chunks, taps,
+    ranks and constants drawn independently (sharing layers agree on the size of a token's values, nothing else)."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice([64, 72, 96, 100, 128, 160, 192])
+    shared, layers = None, []
+    for _ in range(rng.randint(3, 6)):
+        kind = rng.choice(["attention", "latent", "mingru"])
+        if kind == "attention":
+            G = rng.choice([1, 2, 3, 4])
+            H = G * rng.choice([1, 2, 3, 4])
+            d, dv = rng.choice([16, 24, 32, 48, 64]), rng.choice([8, 16, 24, 40, 64])
+            v_mix = rng.random() < 0.7
+            if v_mix and shared is None:
+                shared = (G, dv)
+            elif v_mix:
+                (G, dv), H = shared, shared[0] * rng.choice([1, 2, 4])
+            rot = rng.choice([0, 2, d // 2, d]) // 2 * 2
+            mixer = attention(H, G, d, dv, rng.choice([d ** -0.5, 0.1, 0.3]), chunk=rng.choice([None, 5, 16, 33, 64, 100]),
+                              taps=rng.choice([None, 2, 3, 5]), rot=(rng.choice([100.0, 1e4, 1e6]), rot) if rot else None,
+                              v_mix=v_mix)
+        elif kind == "latent":
+            d, r = rng.choice([8, 16, 24, 32, 64]), rng.choice([2, 4, 8, 16, 32])
+            scaling = (rng.choice([2.0, 4.0, 8.0]), rng.choice([16, 64, 1024]), rng.choice([8.0, 32.0]),
+                       rng.choice([1.0, 2.0])) if rng.random() < 0.7 else None
+            mixer = latent(rng.choice([1, 2, 3, 4, 8]), d, r, rng.choice([8, 16, 24, 32, 64]), rng.choice([12, 16, 32]),
+                           rng.choice([16, 20, 32, 48, 64]), rng.choice([(d + r) ** -0.5, 0.15]),
+                           base=rng.choice([1e3, 1e4, 1e6]), scaling=scaling)
+        else:
+            mixer = mingru(rng.choice([8, 36, 64, 100, 200]))
+        layers.append((mixer, dense(rng.choice([16, 40, 64, 128])) if rng.random() < 0.8 else None))
+    return config(rng.choice([97, 256, 300]), width, layers, taps=rng.choice([0, 1, 2, 3, 4, 5]),
+                  mult=rng.choice([0.25, 0.5, 1.0]), scale=rng.choice([1.0, 2.0, 4.0]), eps=rng.choice([1e-5, 1e-6]))
+
+
 def random_checkpoint(cfg, seed=0):
     return O.random_weights(cfg, seed)
 

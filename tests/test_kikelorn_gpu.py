@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from kikelorn_cases import (Engine, aligned_config, engine_config, mixed_config, odd_config, plain_config,
-                            random_checkpoint, row_error, row_errors)
+                            random_checkpoint, random_config, row_error, row_errors)
 from oracle import kikelorn as O
 
 pytestmark = pytest.mark.gpu
@@ -586,6 +586,26 @@ def test_greedy_generation_through_the_engine(setup):
             # the engine's choice is the oracle's argmax, or lies inside the rounding of the engine's dtype
             assert row.max().item() - row[tok].item() <= (1e-3 if dtype == torch.float32 else 0.1) * spread, (k, tok)
         assert len(out["token_ids"]) == steps
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("seed", [1, 3, 4, 5, 7])
+def test_drawn_configurations(seed, dtype):
+    """Layer orders, sizes and constants drawn from a seed; pages of 64 tokens; prompts whole, then cut and mixed."""
+    cfg = random_config(seed)
+    weights = random_checkpoint(cfg, seed)
+    torch.manual_seed(seed)
+    reqs = {n: torch.randint(0, cfg["vocab"], (L,)).tolist() for n, L in (("a", 230), ("b", 17), ("c", 140), ("d", 2))}
+    want = {n: O.forward(t, weights, cfg).float() for n, t in reqs.items()}
+    engine = Engine(cfg, weights, dtype, blocks=8, slots=3, block_size=64)
+    tol = F32_TOL if dtype == torch.float32 else BF16_TOL
+    for schedule in ([[(n, len(t))] for n, t in reqs.items()],
+                     [[("a", 100), ("b", 3)], [("a", 1), ("b", 14), ("d", 2)], [("a", 65), ("c", 2)], [("c", 1), ("a", 1)],
+                      [("a", 63), ("c", 130)], [("c", 7)]]):
+        got = engine.replay(reqs, schedule)
+        for n in reqs:
+            assert row_error(got[n], want[n]) < tol, (n, row_error(got[n], want[n]))
+    engine.runner.exit()
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
